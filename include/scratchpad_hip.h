@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define SP_ABI_VERSION 11
+#define SP_ABI_VERSION 12
 #define SP_API __attribute__((visibility("default")))
 
 typedef enum { SP_F32 = 0, SP_F16 = 1, SP_BF16 = 2, SP_FP8_E5M2 = 3 /* KV pool only */ } sp_dtype;
@@ -505,13 +505,16 @@ SP_API int sp_stream_add(float* x, int64_t x_stride, const void* a, int64_t a_st
                          const void* c, int64_t c_stride, int64_t num_tokens, int width, int dtype, void* stream);
 
 /* ---- sliding-window attention with pooled blocks (csrc/window_attention.hip) -------------------------------------- */
-/* q [T, heads, dim] rotated in place; k [T, kv_heads, dim] rotated into kpool[loc[t]]; v [T, kv_heads, vdim], every head
- * divided by its root mean square (eps inside the root), into vpool[loc[t]].  Rotation: coordinate i < rot_dims / 2 pairs
- * with i + rot_dims / 2, angle = positions[t] * freq[i] in fp32, cos and sin times mag.                              */
+/* q [T, heads, dim] rotated in place; k [T, kv_heads, dim] rotated into kpool[loc[t]]; v [T, kv_heads, vdim] into
+ * vpool[loc[t]], every head divided by its root mean square (eps inside the root) unless norm_values is 0.  Rotation:
+ * coordinate i < rot_dims / 2 pairs with i + rot_dims / 2 (adjacent = 0) or coordinate 2i with 2i + 1 (adjacent = 1), angle =
+ * positions[t] * freq[i] in fp32, cos and sin times mag.  q_bias [heads * dim], k_bias [kv_heads * dim], v_bias
+ * [kv_heads * vdim] (fp32, each optional, ABI 12) are added before the rotation / the norm.                              */
 SP_API int sp_qkv_rotary_store(void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
                                void* kpool, int64_t kp_stride, void* vpool, int64_t vp_stride, const int64_t* positions,
-                               const int64_t* loc, const float* freq, float mag, int64_t num_tokens, int heads, int kv_heads,
-                               int dim, int vdim, int rot_dims, float eps, int dtype, void* stream);
+                               const int64_t* loc, const float* freq, float mag, const float* q_bias, const float* k_bias,
+                               const float* v_bias, int64_t num_tokens, int heads, int kv_heads, int dim, int vdim,
+                               int rot_dims, int adjacent, int norm_values, float eps, int dtype, void* stream);
 /* every token of the step whose position + 1 is a multiple of `block` writes the mean of the last `block` cached key rows
  * (value rows) of its request into kpooled (vpooled) at its own slot; run after the step's rows are in the pool       */
 SP_API int sp_pool_blocks(void* kpooled, void* vpooled, const void* kpool, const void* vpool, int64_t kp_stride,
@@ -520,13 +523,15 @@ SP_API int sp_pool_blocks(void* kpooled, void* vpooled, const void* kpool, const
 /* out [T, heads, vdim]: a query at position p attends, in one fp32 softmax of (q . k) * scale, to the cached tokens j with
  * 0 <= p - j < window and to the pooled rows of the blocks b with b * block + block - 1 <= p - window.  window <= 0: every
  * earlier token and no blocks; block <= 0: no blocks.  Query head h reads key/value head h / (heads / kv_heads).
- * vdim <= 256.  matrix != 0: steps that bring portions of prompts in a 16-bit type, with dim and vdim of 64 or 128, run on
- * the matrix cores (16 tokens x one key/value head per workgroup); everything else on the fp32 vector kernel.         */
+ * vdim <= 256.  sinks (fp32 [heads], optional, ABI 12): the softmax's denominator of head h also holds exp(sinks[h]) - a
+ * term without a key or a value, not scaled.  matrix != 0: steps that bring portions of prompts in a 16-bit type, with dim
+ * and vdim of 64 or 128, run on the matrix cores (16 tokens x one key/value head per workgroup); everything else on the
+ * fp32 vector kernel.                                                                                                  */
 SP_API int sp_window_attention(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kpool,
                                const void* vpool, const void* kpooled, const void* vpooled, int64_t kp_stride,
                                int64_t vp_stride, const int32_t* req_to_token, int64_t table_stride, int64_t num_tokens,
                                int heads, int kv_heads, int dim, int vdim, int64_t window, int block, float scale,
-                               int matrix, SP_SEQ_PARAMS, int dtype, void* stream);
+                               const float* sinks, int matrix, SP_SEQ_PARAMS, int dtype, void* stream);
 
 /* ---- state-space and matrix-memory recurrences (csrc/ssm.hip, csrc/mlstm.hip) -------------------------------------- */
 /* out[t, j] = bias[j] + sum_i weight[j, i] x[t, i]: fp32 weights, accumulation and output (x in `dtype`; bias optional) */
@@ -559,6 +564,52 @@ SP_API int sp_mlstm_scan(void* out, int64_t out_stride, const void* q, int64_t q
                          const float* fpre, const float* norm_w, float* S_state, int64_t S_stride, float* n_state,
                          int64_t n_stride, float* m_state, int64_t m_stride, int heads, int dim, int vdim, float cap,
                          float eps, SP_SEQ_PARAMS, int dtype, void* stream);
+
+/* ================================================================================================================
+ * ABI 12: sublayer results that are gated and normed before they join the fp32 stream, the generalized delta rule, a
+ * linear attention whose forget gate also writes, squared ReLU, scaled and soft-capped logits.
+ */
+/* Tail of a sublayer, one pass per row (N = division by the row's root mean square, eps inside the root):
+ *   y = a                               or, with a second branch b,   y = (N(a) wa + N(b) wb) / 2
+ *   y = y * sigmoid(gate + gate_bias)   (gate optional; gate_bias optional)
+ *   x = x + N(y) weight                 (x fp32, in place)
+ *   x = x + extra                       (extra fp32, optional)
+ *   out_next = N(x) next_weight         (optional, in `dtype`: the next sublayer's input)
+ * a, b, gate in `dtype` with their row strides; every weight fp32 [width].  width <= 15360.                           */
+SP_API int sp_gated_add_norm(float* x, int64_t x_stride, const void* a, int64_t a_stride, const float* wa, const void* b,
+                             int64_t b_stride, const float* wb, const void* gate, int64_t gate_stride,
+                             const float* gate_bias, const float* weight, const float* extra, int64_t extra_stride,
+                             void* out_next, int64_t next_stride, const float* next_weight, int64_t num_tokens, int width,
+                             float eps, int dtype, void* stream);
+/* out[t, j] = max(x[t, j], 0)^2 */
+SP_API int sp_relu_square(void* out, const void* x, int64_t num_tokens, int d, int64_t x_stride, int64_t out_stride,
+                          int dtype, void* stream);
+/* out[r, j] = cap * tanh(logits[r, j] * scale / cap), or logits * scale when cap <= 0; out fp32, logits in `dtype` */
+SP_API int sp_scale_softcap(float* out, int64_t out_stride, const void* logits, int64_t row_stride, int64_t rows, int n,
+                            float scale, float cap, int dtype, void* stream);
+/* Gates of the generalized delta rule, fp32 [T, channels]:
+ *   decay[t, c]  = exp(-rate * sigmoid(sum_r w2t[r, c] * tanh(p[t, r]) + w0[c]))     (p [T, rank] in `dtype`)
+ *   remove[t, c] = sigmoid(apre[t, c] + a_bias[c])                                   (apre in `dtype`)                */
+SP_API int sp_delta_gates(float* decay, float* remove, const void* p, int64_t p_stride, const float* w2t, const float* w0,
+                          const void* apre, int64_t a_stride, const float* a_bias, int64_t num_tokens, int channels, int rank,
+                          float rate, int dtype, void* stream);
+/* Per (request, head) over the request's rows of this step in order, S [head_dim(key), head_dim(value)] fp32 from
+ * state[request slot] (zeros at a sequence's first token) and back:
+ *   u = k / sqrt(|k|^2 + 1e-6);  S = diag(decay) S - (remove * u)(u^T S) + k v^T (both terms on the previous S);  o = S^T r
+ *   out = o / rms_head(o) * norm_w * sigmoid(g).   r, k, v, g, out in `dtype`; decay, remove fp32 [T, heads * head_dim].
+ * head_dim <= 256.                                                                                                    */
+SP_API int sp_delta_recurrence(void* out, int64_t out_stride, const void* r, int64_t r_stride, const void* k,
+                               int64_t k_stride, const void* v, int64_t v_stride, const void* g, int64_t g_stride,
+                               const float* decay, const float* remove, const float* norm_w, float* state,
+                               int64_t state_stride, int heads, int head_dim, float eps, SP_SEQ_PARAMS, int dtype,
+                               void* stream);
+/* Per (request, head) over the request's rows in order, S [dim, vdim] fp32 from state[request slot] and back:
+ *   q = silu(qpre);  f = lower + (1 - lower) sigmoid(fpre + f_bias);  S = diag(f) S + (1 - f) v^T;  o = S^T q
+ *   out = o / rms_head(o) * norm_w   (norm_w [vdim], shared by the heads).  dim, vdim <= 256.                          */
+SP_API int sp_hgrn2_scan(void* out, int64_t out_stride, const void* qpre, int64_t q_stride, const void* fpre,
+                         int64_t f_stride, const void* v, int64_t v_stride, const float* f_bias, const float* lower,
+                         const float* norm_w, float* state, int64_t state_stride, int heads, int dim, int vdim, float eps,
+                         SP_SEQ_PARAMS, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -130,17 +130,27 @@ SIGNATURES = {
     "sp_norm_shift": (_i32, [_vp, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i32, _f32, *_SEQ, _i32, _vp]),
     "sp_norm_save_last": (_i32, [_vp, _i64, _vp, _i64, _vp, _i32, _f32, *_SEQ, _vp]),
     "sp_stream_add": (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _i32, _i32, _vp]),
-    "sp_qkv_rotary_store": (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _f32, _i64, _i32,
-                                   _i32, _i32, _i32, _i32, _f32, _i32, _vp]),
+    "sp_qkv_rotary_store": (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _f32, _vp, _vp, _vp,
+                                   _i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _vp]),
     "sp_pool_blocks": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i32, _i32, _i32, *_SEQ, _i32, _vp]),
     "sp_window_attention": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i32, _i32, _i32,
-                                   _i32, _i64, _i32, _f32, _i32, *_SEQ, _i32, _vp]),
+                                   _i32, _i64, _i32, _f32, _vp, _i32, *_SEQ, _i32, _vp]),
     "sp_small_linear_f32": (_i32, [_vp, _vp, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _vp]),
     "sp_causal_conv_silu": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i32, _i32, *_SEQ, _i32, _vp]),
     "sp_mamba2_scan": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, *_SEQ, _i32, _vp]),
     "sp_gated_group_norm": (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _i32, _i32, _f32, _i32, _vp]),
     "sp_mlstm_scan": (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp,
                              _i64, _i32, _i32, _i32, _f32, _f32, *_SEQ, _i32, _vp]),
+    # ---- ABI 12
+    "sp_gated_add_norm": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _i64, _vp, _vp, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _vp,
+                                 _i64, _i32, _f32, _i32, _vp]),
+    "sp_relu_square": (_i32, [_vp, _vp, _i64, _i32, _i64, _i64, _i32, _vp]),
+    "sp_scale_softcap": (_i32, [_vp, _i64, _vp, _i64, _i64, _i32, _f32, _f32, _i32, _vp]),
+    "sp_delta_gates": (_i32, [_vp, _vp, _vp, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _i32, _i32, _f32, _i32, _vp]),
+    "sp_delta_recurrence": (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i32, _i32,
+                                   _f32, *_SEQ, _i32, _vp]),
+    "sp_hgrn2_scan": (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _f32,
+                             *_SEQ, _i32, _vp]),
 }
 
 
@@ -174,7 +184,7 @@ def load() -> ctypes.CDLL:
             continue
         fn.restype = res
         fn.argtypes = args
-    if lib.sp_abi_version() != 11:
+    if lib.sp_abi_version() != 12:
         raise RuntimeError("libscratchpad_hip.so ABI version mismatch")
     _lib = lib
     return lib
@@ -1255,8 +1265,12 @@ def stream_add(x: torch.Tensor, a: torch.Tensor, b: Optional[torch.Tensor] = Non
 
 def qkv_rotary_store(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor,
                      positions: torch.Tensor, loc: torch.Tensor, freq: Optional[torch.Tensor], mag: float, heads: int,
-                     kv_heads: int, dim: int, vdim: int, eps: float) -> None:
-    """q [T, heads * dim] rotated in place; k rotated, v head-normed into the pools' rows loc (views: strides are taken)"""
+                     kv_heads: int, dim: int, vdim: int, eps: float, adjacent: bool = False, norm_values: bool = True,
+                     q_bias: Optional[torch.Tensor] = None, k_bias: Optional[torch.Tensor] = None,
+                     v_bias: Optional[torch.Tensor] = None) -> None:
+    """q [T, heads * dim] rotated in place; k rotated, v (head-normed unless ``norm_values`` is off) into the pools' rows
+    loc (views: strides are taken).  ``adjacent``: coordinate 2i pairs with 2i + 1 instead of i with i + dims / 2.  fp32
+    biases, where given, are added before the rotation / the norm."""
     for name, t, n in (("q", q, heads * dim), ("k", k, kv_heads * dim), ("v", v, kv_heads * vdim)):
         if _mat(t, name).shape[1] != n or t.dtype != q.dtype or t.shape[0] != q.shape[0]:
             raise RuntimeError(f"qkv_rotary_store: {name} must be [T, {n}]")
@@ -1265,10 +1279,14 @@ def qkv_rotary_store(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, kpool: t
         raise RuntimeError("qkv_rotary_store: pools [P, kv_heads * dim] / [P, kv_heads * vdim] of q's dtype")
     if positions.dtype != torch.int64 or loc.dtype != torch.int64 or loc.shape[0] != q.shape[0] or positions.shape[0] != q.shape[0]:
         raise RuntimeError("qkv_rotary_store: int64 positions and loc, one per row")
+    for name, t, n in (("q_bias", q_bias, heads * dim), ("k_bias", k_bias, kv_heads * dim), ("v_bias", v_bias, kv_heads * vdim)):
+        if t is not None and _f32(t, name).numel() != n:
+            raise RuntimeError(f"qkv_rotary_store: {name} must hold {n} values")
     dims = 0 if freq is None else 2 * _f32(freq, "freq").shape[0]
     _check(load().sp_qkv_rotary_store(q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
                                       kpool.data_ptr(), kpool.stride(0), vpool.data_ptr(), vpool.stride(0), positions.data_ptr(),
-                                      loc.data_ptr(), _ptr(freq), mag, q.shape[0], heads, kv_heads, dim, vdim, dims, eps, _dt(q),
+                                      loc.data_ptr(), _ptr(freq), mag, _ptr(q_bias), _ptr(k_bias), _ptr(v_bias), q.shape[0],
+                                      heads, kv_heads, dim, vdim, dims, int(adjacent), int(norm_values), eps, _dt(q),
                                       _stream()), "sp_qkv_rotary_store")
 
 
@@ -1284,9 +1302,10 @@ def pool_blocks(kpooled: torch.Tensor, vpooled: torch.Tensor, kpool: torch.Tenso
 
 def window_attention(q: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, kpooled: Optional[torch.Tensor],
                      vpooled: Optional[torch.Tensor], req_to_token: torch.Tensor, seq: SeqParams, heads: int, kv_heads: int,
-                     dim: int, vdim: int, window: int, block: int, scale: float, matrix: bool = True) -> torch.Tensor:
+                     dim: int, vdim: int, window: int, block: int, scale: float, matrix: bool = True,
+                     sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """q [T, heads * dim] (rotated) -> [T, heads * vdim]; matrix=False keeps 16-bit prompt portions off the matrix-core
-    kernel (comparisons)"""
+    kernel (comparisons); sinks fp32 [heads]: one more term exp(sink) in every softmax's denominator"""
     _mat(q, "q"), _mat(kpool, "kpool"), _mat(vpool, "vpool")
     T = q.shape[0]
     if q.shape[1] != heads * dim or kpool.shape[1] != kv_heads * dim or vpool.shape[1] != kv_heads * vdim or \
@@ -1294,11 +1313,14 @@ def window_attention(q: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, 
         raise RuntimeError("window_attention: shapes / dtypes do not fit")
     if kpooled is not None and (kpooled.stride(0) != kpool.stride(0) or vpooled.stride(0) != vpool.stride(0)):
         raise RuntimeError("window_attention: pooled buffers must mirror the token buffers")
+    if sinks is not None and _f32(sinks, "sinks").numel() != heads:
+        raise RuntimeError("window_attention: sinks must hold one value per query head")
     out = empty_rows(T, heads * vdim, q.dtype, q.device)
     _check(load().sp_window_attention(out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), kpool.data_ptr(),
                                       vpool.data_ptr(), _ptr(kpooled), _ptr(vpooled), kpool.stride(0), vpool.stride(0),
                                       req_to_token.data_ptr(), req_to_token.stride(0), T, heads, kv_heads, dim, vdim,
-                                      window, block, scale, int(matrix), *seq.args, _dt(q), _stream()), "sp_window_attention")
+                                      window, block, scale, _ptr(sinks), int(matrix), *seq.args, _dt(q), _stream()),
+           "sp_window_attention")
     return out
 
 
@@ -1379,4 +1401,108 @@ def mlstm_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tenso
                                 v.data_ptr(), v.stride(0), g.data_ptr(), g.stride(0), ipre.data_ptr(), fpre.data_ptr(),
                                 norm_w.data_ptr(), S.data_ptr(), S.stride(0), n.data_ptr(), n.stride(0), m.data_ptr(),
                                 m.stride(0), heads, dim, vdim, cap, eps, *seq.args, _dt(q), _stream()), "sp_mlstm_scan")
+    return out
+
+
+# --------------------------------------------------------------------------- gated normed sublayer results, delta rule, forget-write scan
+def gated_add_norm(x: torch.Tensor, a: torch.Tensor, weight: torch.Tensor, eps: float, gate: Optional[torch.Tensor] = None,
+                   gate_bias: Optional[torch.Tensor] = None, b: Optional[torch.Tensor] = None, wa: Optional[torch.Tensor] = None,
+                   wb: Optional[torch.Tensor] = None, extra: Optional[torch.Tensor] = None,
+                   next_weight: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """x fp32 [T, W] += N(y * sigmoid(gate + gate_bias)) * weight in place, y = a, or (N(a) wa + N(b) wb) / 2 with a second
+    branch; then x += extra (fp32); with ``next_weight`` returns N(x) * next_weight in a's dtype (the next sublayer's
+    input).  a, b, gate may be views (their row strides are taken)."""
+    _mat(x, "x"), _mat(a, "a"), _f32(weight, "weight")
+    T, W = x.shape
+    if x.dtype != torch.float32 or a.shape != (T, W) or weight.numel() != W:
+        raise RuntimeError("gated_add_norm: x fp32 [T, W], a [T, W], weight [W]")
+    for name, t in (("b", b), ("gate", gate)):
+        if t is not None and (_mat(t, name).shape != (T, W) or t.dtype != a.dtype):
+            raise RuntimeError(f"gated_add_norm: {name} must be [T, W] of a's dtype")
+    if b is not None and (wa is None or wb is None or _f32(wa, "wa").numel() != W or _f32(wb, "wb").numel() != W):
+        raise RuntimeError("gated_add_norm: two branches need their norm weights wa, wb [W]")
+    if gate_bias is not None and _f32(gate_bias, "gate_bias").numel() != W:
+        raise RuntimeError("gated_add_norm: gate_bias [W]")
+    if extra is not None and (_mat(extra, "extra").shape != (T, W) or extra.dtype != torch.float32):
+        raise RuntimeError("gated_add_norm: extra fp32 [T, W]")
+    nxt = None
+    if next_weight is not None:
+        if _f32(next_weight, "next_weight").numel() != W:
+            raise RuntimeError("gated_add_norm: next_weight [W]")
+        nxt = empty_rows(T, W, a.dtype, x.device)
+    _check(load().sp_gated_add_norm(x.data_ptr(), x.stride(0), a.data_ptr(), a.stride(0), _ptr(wa), _ptr(b),
+                                    0 if b is None else b.stride(0), _ptr(wb), _ptr(gate), 0 if gate is None else gate.stride(0),
+                                    _ptr(gate_bias), weight.data_ptr(), _ptr(extra), 0 if extra is None else extra.stride(0),
+                                    _ptr(nxt), 0 if nxt is None else nxt.stride(0), _ptr(next_weight), T, W, eps, _dt(a),
+                                    _stream()), "sp_gated_add_norm")
+    return nxt
+
+
+def relu_square(x: torch.Tensor) -> torch.Tensor:
+    """max(x, 0)^2 of x [T, d] (a view: its row stride is taken)"""
+    _mat(x, "x")
+    out = empty_rows(x.shape[0], x.shape[1], x.dtype, x.device)
+    _check(load().sp_relu_square(out.data_ptr(), x.data_ptr(), x.shape[0], x.shape[1], x.stride(0), out.stride(0), _dt(x),
+                                 _stream()), "sp_relu_square")
+    return out
+
+
+def scale_softcap(logits: torch.Tensor, scale: float, cap: float) -> torch.Tensor:
+    """fp32 [rows, n] = cap * tanh(logits * scale / cap) (cap 0 or less: logits * scale)"""
+    _mat(logits, "logits")
+    out = torch.empty(logits.shape, dtype=torch.float32, device=logits.device)
+    _check(load().sp_scale_softcap(out.data_ptr(), out.stride(0), logits.data_ptr(), logits.stride(0), logits.shape[0],
+                                   logits.shape[1], scale, cap or 0.0, _dt(logits), _stream()), "sp_scale_softcap")
+    return out
+
+
+def delta_gates(p: torch.Tensor, w2t: torch.Tensor, w0: torch.Tensor, apre: torch.Tensor, a_bias: torch.Tensor, rate: float):
+    """(decay, remove) fp32 [T, channels]: exp(-rate * sigmoid(tanh(p) w2t + w0)) and sigmoid(apre + a_bias)"""
+    _mat(p, "p"), _mat(apre, "apre"), _f32(w2t, "w2t"), _f32(w0, "w0"), _f32(a_bias, "a_bias")
+    T, n = apre.shape
+    if w2t.shape != (p.shape[1], n) or w0.numel() != n or a_bias.numel() != n or p.shape[0] != T or p.dtype != apre.dtype:
+        raise RuntimeError("delta_gates: p [T, rank], w2t [rank, channels], w0, a_bias [channels], apre [T, channels]")
+    decay = torch.empty((T, n), dtype=torch.float32, device=p.device)
+    remove = torch.empty((T, n), dtype=torch.float32, device=p.device)
+    _check(load().sp_delta_gates(decay.data_ptr(), remove.data_ptr(), p.data_ptr(), p.stride(0), w2t.data_ptr(), w0.data_ptr(),
+                                 apre.data_ptr(), apre.stride(0), a_bias.data_ptr(), T, n, p.shape[1], rate, _dt(p), _stream()),
+           "sp_delta_gates")
+    return decay, remove
+
+
+def delta_recurrence(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, g: torch.Tensor, decay: torch.Tensor,
+                     remove: torch.Tensor, norm_w: torch.Tensor, state: torch.Tensor, seq: SeqParams, heads: int, dim: int,
+                     eps: float) -> torch.Tensor:
+    """r, k, v, g [T, heads * dim] (views) -> [T, heads * dim]; state [slots, heads, dim, dim] fp32 is read and moved on"""
+    T, n = seq.num_tokens, heads * dim
+    for name, t in (("r", r), ("k", k), ("v", v), ("g", g)):
+        if _mat(t, name).shape != (T, n) or t.dtype != r.dtype:
+            raise RuntimeError(f"delta_recurrence: {name} must be [num_tokens, heads * dim] of one dtype")
+    _f32(decay, "decay"), _f32(remove, "remove"), _f32(norm_w, "norm_w"), _f32(state, "state")
+    if decay.shape != (T, n) or remove.shape != (T, n) or norm_w.numel() != n or state.shape[1:] != (heads, dim, dim):
+        raise RuntimeError("delta_recurrence: decay, remove [T, H*D], norm_w [H*D], state [slots, H, D, D]")
+    out = empty_rows(T, n, r.dtype, r.device)
+    _check(load().sp_delta_recurrence(out.data_ptr(), out.stride(0), r.data_ptr(), r.stride(0), k.data_ptr(), k.stride(0),
+                                      v.data_ptr(), v.stride(0), g.data_ptr(), g.stride(0), decay.data_ptr(), remove.data_ptr(),
+                                      norm_w.data_ptr(), state.data_ptr(), state.stride(0), heads, dim, eps, *seq.args,
+                                      _dt(r), _stream()), "sp_delta_recurrence")
+    return out
+
+
+def hgrn2_scan(qpre: torch.Tensor, fpre: torch.Tensor, v: torch.Tensor, f_bias: torch.Tensor, lower: torch.Tensor,
+               norm_w: torch.Tensor, state: torch.Tensor, seq: SeqParams, heads: int, dim: int, vdim: int, eps: float) -> torch.Tensor:
+    """qpre, fpre [T, heads * dim], v [T, heads * vdim] (views) -> [T, heads * vdim]; state [slots, heads, dim, vdim] fp32"""
+    T = seq.num_tokens
+    for name, t, w in (("qpre", qpre, heads * dim), ("fpre", fpre, heads * dim), ("v", v, heads * vdim)):
+        if _mat(t, name).shape != (T, w) or t.dtype != qpre.dtype:
+            raise RuntimeError(f"hgrn2_scan: {name} must be [num_tokens, {w}] of one dtype")
+    _f32(f_bias, "f_bias"), _f32(lower, "lower"), _f32(norm_w, "norm_w"), _f32(state, "state")
+    if f_bias.numel() != heads * dim or lower.numel() != heads * dim or norm_w.numel() != vdim or \
+            state.shape[1:] != (heads, dim, vdim):
+        raise RuntimeError("hgrn2_scan: f_bias, lower [H*D], norm_w [vdim], state [slots, H, D, vdim]")
+    out = empty_rows(T, heads * vdim, qpre.dtype, qpre.device)
+    _check(load().sp_hgrn2_scan(out.data_ptr(), out.stride(0), qpre.data_ptr(), qpre.stride(0), fpre.data_ptr(), fpre.stride(0),
+                                v.data_ptr(), v.stride(0), f_bias.data_ptr(), lower.data_ptr(), norm_w.data_ptr(),
+                                state.data_ptr(), state.stride(0), heads, dim, vdim, eps, *seq.args, _dt(qpre), _stream()),
+           "sp_hgrn2_scan")
     return out

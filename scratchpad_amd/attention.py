@@ -536,10 +536,13 @@ class LatentAttention(nn.Module):
 class PooledWindowAttention(nn.Module):
     """Layer-local constants of a grouped-query attention layer over a WindowKVPool: a query sees the ``window`` latest
     tokens and, for every block of ``block`` positions wholly behind the window, the block's mean key and value (one
-    softmax over both); key width ``dim`` and value width ``vdim`` may differ.  window None: plain causal attention."""
+    softmax over both); key width ``dim`` and value width ``vdim`` may differ.  window None: plain causal attention.
+    ``sinks``: one learned fp32 number per query head whose exponential joins the softmax's denominator (a key every query
+    sees, without a value).  ``norm_values``: the cache holds every value head divided by its root mean square.  q, k, v may
+    carry fp32 biases (``store``), added before the rotation."""
 
     def __init__(self, num_heads: int, num_kv_heads: int, dim: int, vdim: int, scaling: float, layer_id: int,
-                 window: Optional[int] = None, block: Optional[int] = None):
+                 window: Optional[int] = None, block: Optional[int] = None, sinks: bool = False, norm_values: bool = True):
         super().__init__()
         if num_heads % num_kv_heads:
             raise ValueError("query heads must be a multiple of key/value heads")
@@ -547,14 +550,19 @@ class PooledWindowAttention(nn.Module):
         self.dim, self.vdim, self.scaling, self.layer_id = dim, vdim, scaling, layer_id
         self.window = int(window) if window else 0
         self.block = int(block) if (block and window) else 0
+        self.norm_values = norm_values
+        self.sinks = nn.Parameter(torch.zeros(num_heads, dtype=torch.float32), requires_grad=False) if sinks else None
 
-    def store(self, q, k, v, rotary, positions, eps: float, forward_batch: "ForwardBatch") -> None:
-        """rotate q in place; rotate k, norm v per head and put both into the pool; then the blocks this step completes"""
-        forward_batch.attn_backend.store_window(q, k, v, rotary, positions, eps, self, forward_batch)
+    def store(self, q, k, v, rotary, positions, eps: float, forward_batch: "ForwardBatch", cache_id: Optional[int] = None,
+              biases=(None, None, None)) -> None:
+        """rotate q in place; rotate k, norm v per head (if the layer does) and put both into the pool; then the blocks this
+        step completes.  ``cache_id``: the pool layer to use instead of ``layer_id`` (a layer that runs several times on the
+        same weights keeps one cache per run)."""
+        forward_batch.attn_backend.store_window(q, k, v, rotary, positions, eps, self, forward_batch, cache_id, biases)
 
-    def forward(self, q, forward_batch: "ForwardBatch"):
+    def forward(self, q, forward_batch: "ForwardBatch", cache_id: Optional[int] = None):
         """q [T, heads * dim] (rotated) -> [T, heads * vdim]; the step's rows are in the pool"""
-        return forward_batch.attn_backend.forward_window(q, self, forward_batch)
+        return forward_batch.attn_backend.forward_window(q, self, forward_batch, cache_id)
 
 
 class SequenceBackend(AttentionBackend):
@@ -599,23 +607,29 @@ class SequenceBackend(AttentionBackend):
         return _native.latent_attention(q_lat, q_rot, pool, forward_batch.req_to_token_pool.req_to_token, self.seq,
                                         layer.scaling)
 
-    def store_window(self, q, k, v, rotary, positions, eps, layer: "PooledWindowAttention", forward_batch: "ForwardBatch"):
+    def store_window(self, q, k, v, rotary, positions, eps, layer: "PooledWindowAttention", forward_batch: "ForwardBatch",
+                     cache_id=None, biases=(None, None, None)):
         pool = forward_batch.token_to_kv_pool
-        kbuf, vbuf = pool.get_kv_buffer(layer.layer_id)
+        cache = layer.layer_id if cache_id is None else cache_id
+        kbuf, vbuf = pool.get_kv_buffer(cache)
         freq, mag = (rotary.freq, rotary.magnitude) if rotary is not None else (None, 1.0)
         _native.qkv_rotary_store(q, k, v, kbuf, vbuf, positions, forward_batch.out_cache_loc, freq, mag, layer.tp_q_head_num,
-                                 layer.tp_k_head_num, layer.dim, layer.vdim, eps)
+                                 layer.tp_k_head_num, layer.dim, layer.vdim, eps,
+                                 adjacent=bool(rotary is not None and rotary.adjacent_pairs), norm_values=layer.norm_values,
+                                 q_bias=biases[0], k_bias=biases[1], v_bias=biases[2])
         if layer.block:
-            kp, vp = pool.get_pooled_buffers(layer.layer_id)
+            kp, vp = pool.get_pooled_buffers(cache)
             _native.pool_blocks(kp, vp, kbuf, vbuf, forward_batch.req_to_token_pool.req_to_token, self.seq, layer.block)
 
-    def forward_window(self, q, layer: "PooledWindowAttention", forward_batch: "ForwardBatch"):
+    def forward_window(self, q, layer: "PooledWindowAttention", forward_batch: "ForwardBatch", cache_id=None):
         pool = forward_batch.token_to_kv_pool
-        kbuf, vbuf = pool.get_kv_buffer(layer.layer_id)
-        kp, vp = pool.get_pooled_buffers(layer.layer_id) if layer.block else (None, None)
+        cache = layer.layer_id if cache_id is None else cache_id
+        kbuf, vbuf = pool.get_kv_buffer(cache)
+        kp, vp = pool.get_pooled_buffers(cache) if layer.block else (None, None)
         return _native.window_attention(q, kbuf, vbuf, kp, vp, forward_batch.req_to_token_pool.req_to_token, self.seq,
                                         layer.tp_q_head_num, layer.tp_k_head_num, layer.dim, layer.vdim, layer.window,
-                                        layer.block, layer.scaling)
+                                        layer.block, layer.scaling,
+                                        sinks=None if layer.sinks is None else layer.sinks.data)
 
     def forward_decode(self, q, k, v, layer, forward_batch, save_kv_cache: bool = True):
         raise NotImplementedError("this backend serves latent attention layers (forward_latent) and windowed ones (forward_window)")

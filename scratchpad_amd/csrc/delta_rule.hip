@@ -1,0 +1,209 @@
+// Generalized delta rule: a per-head matrix state with a per-channel decay and a per-channel removal along the unit key.
+// Per head, with r, k, v of a token, decay w and removal rate a per key channel, all of the recurrence in fp32:
+//   u  = k / sqrt(|k|^2 + 1e-6)
+//   S' = diag(w) S - (a * u) (u^T S) + k v^T            (both first terms read the state the previous token left)
+//   o  = S'^T r
+//   out = o / rms_head(o) * norm_w * sigmoid(g)
+// The gates come from sp_delta_gates:
+//   w = exp(-rate * sigmoid(W2 tanh(p) + w0))            (p = the low-rank projection's output)
+//   a = sigmoid(apre + a_bias)
+//
+// One workgroup per (request, head): a column of S (one value channel) lives in the registers of 1, 2 or 4 neighbouring
+// lanes; the request's tokens of this step are walked in order from the state the previous step left in the pool (zeros
+// at a sequence's first token), staged through LDS in passes.  A token costs two sweeps over the column - u^T S first,
+// then the update with the numerator - and two lane exchanges, no workgroup barrier.  Prompt portions and single decoded
+// tokens take the same path, and the order of every sum depends on the head only.
+#include "seq_batch.h"
+
+namespace sp {
+namespace {
+
+// w2t: [rank, channels] fp32 (the up-projection transposed: neighbouring threads read neighbouring channels)
+template <typename Tag>
+__global__ void __launch_bounds__(kBlock)
+delta_gates_kernel(float* decay, float* remove, const void* p, int64_t p_stride, const float* w2t, const float* w0,
+                   const void* apre, int64_t a_stride, const float* a_bias, int channels, int rank, float rate) {
+  typedef Elem<Tag> E;
+  extern __shared__ float tp[];
+  const int64_t t = blockIdx.x;
+  for (int r = threadIdx.x; r < rank; r += blockDim.x) tp[r] = tanhf(E::load(p, t * p_stride + r));
+  __syncthreads();
+  for (int c = threadIdx.x; c < channels; c += blockDim.x) {
+    float acc = 0.f;
+    for (int r = 0; r < rank; ++r) acc += w2t[(int64_t)r * channels + c] * tp[r];
+    acc += w0[c];
+    decay[t * channels + c] = expf(-rate / (1.f + expf(-acc)));
+    const float z = E::load(apre, t * a_stride + c) + a_bias[c];
+    remove[t * channels + c] = 1.f / (1.f + expf(-z));
+  }
+}
+
+constexpr int delta_chunk(int KP) { return KP > 64 ? 8 : 16; }                      // tokens staged in LDS per pass
+constexpr int delta_split(int KP) { return KP > 64 ? 4 : (KP > 32 ? 2 : 1); }       // lanes that share one column of S
+
+// thread = (column col of S, part): part p of SP owns the rows [p DS, (p + 1) DS) of the column.  LDS rows are padded by
+// 4 floats per part so that the parts' simultaneous broadcast reads fall into different banks.
+template <typename Tag, int KP>
+__global__ void __launch_bounds__(KP * delta_split(KP) < 64 ? 64 : KP * delta_split(KP))
+delta_recurrence_kernel(void* out, int64_t out_stride, const void* r, int64_t r_stride, const void* k, int64_t k_stride,
+                        const void* v, int64_t v_stride, const void* g, int64_t g_stride, const float* decay,
+                        const float* remove, const float* norm_w, float* state, int64_t state_stride, SeqBatch s, int H,
+                        int K, float eps) {
+  typedef Elem<Tag> E;
+  constexpr int kChunk = delta_chunk(KP), SP = delta_split(KP), DS = KP / SP, ROW = KP + 4 * SP;
+  __shared__ float sr[kChunk][ROW], sk[kChunk][ROW], sw[kChunk][ROW], su[kChunk][ROW], sau[kChunk][ROW];
+  __shared__ float sv[kChunk][KP], so[kChunk][KP], sinv[kChunk];
+  const int b = blockIdx.x, h = blockIdx.y, j = threadIdx.x;
+  const int nthreads = blockDim.x, wave = j >> 6, lane = j & 63, waves = nthreads >> 6;
+  const int col = j / SP, part = j % SP;
+  int64_t start, len, prefix;
+  seq_span(s, b, start, len, prefix);
+  if (len <= 0) return;
+  const bool live = col < K;
+  float* st = state + load_idx(s.req_pool_indices, b, s.idx64) * state_stride + (int64_t)h * K * K;
+  const bool held = prefix > 0;
+  float S[DS];
+#pragma unroll
+  for (int ii = 0; ii < DS; ++ii) {
+    const int i = part * DS + ii;
+    S[ii] = (live && i < K && held) ? st[(int64_t)i * K + col] : 0.f;
+  }
+  const int64_t hc = (int64_t)h * K, HK = (int64_t)H * K;
+  const int mine = part * (DS + 4);
+  for (int64_t c0 = 0; c0 < len; c0 += kChunk) {
+    const int n = (int)(len - c0 < kChunk ? len - c0 : kChunk);
+    __syncthreads();
+    for (int e = j; e < n * KP; e += nthreads) {
+      const int tt = e / KP, i = e % KP;
+      const int64_t row = start + c0 + tt;
+      const bool ok = i < K;
+      const int at = i + 4 * (i / DS);
+      sr[tt][at] = ok ? E::load(r, row * r_stride + hc + i) : 0.f;
+      sk[tt][at] = ok ? E::load(k, row * k_stride + hc + i) : 0.f;
+      sw[tt][at] = ok ? decay[row * HK + hc + i] : 0.f;
+      sau[tt][at] = ok ? remove[row * HK + hc + i] : 0.f;
+      sv[tt][i] = ok ? E::load(v, row * v_stride + hc + i) : 0.f;
+    }
+    __syncthreads();
+    // the unit key of every token of the pass: a wave per token
+    for (int tt = wave; tt < n; tt += waves) {
+      float ss = 0.f;
+      for (int i = lane; i < K; i += 64) {
+        const float x = sk[tt][i + 4 * (i / DS)];
+        ss += x * x;
+      }
+      ss = wave_sum(ss);
+      const float inv = 1.f / sqrtf(ss + 1e-6f);
+      for (int i = lane; i < KP; i += 64) {
+        const int at = i + 4 * (i / DS);
+        const float uu = sk[tt][at] * inv;
+        su[tt][at] = uu;
+        sau[tt][at] *= uu;
+      }
+    }
+    __syncthreads();
+    for (int tt = 0; tt < n; ++tt) {
+      const float* pu = &su[tt][mine];
+      const float* pau = &sau[tt][mine];
+      const float* pw = &sw[tt][mine];
+      const float* pk = &sk[tt][mine];
+      const float* pr = &sr[tt][mine];
+      float proj = 0.f;
+#pragma unroll
+      for (int ii = 0; ii < DS; ++ii) proj += pu[ii] * S[ii];
+#pragma unroll
+      for (int off = 1; off < SP; off <<= 1) proj += __shfl_xor(proj, off, 64);
+      const float vj = live ? sv[tt][col] : 0.f;
+      float num = 0.f;
+#pragma unroll
+      for (int ii = 0; ii < DS; ++ii) {
+        S[ii] = pw[ii] * S[ii] - pau[ii] * proj + pk[ii] * vj;
+        num += S[ii] * pr[ii];
+      }
+#pragma unroll
+      for (int off = 1; off < SP; off <<= 1) num += __shfl_xor(num, off, 64);
+      if (live && part == 0) so[tt][col] = num;
+    }
+    __syncthreads();
+    // per-head RMS of o, output weight and gate
+    for (int tt = wave; tt < n; tt += waves) {
+      float ss = 0.f;
+      for (int i = lane; i < K; i += 64) ss += so[tt][i] * so[tt][i];
+      ss = wave_sum(ss);
+      if (lane == 0) sinv[tt] = 1.f / sqrtf(ss / (float)K + eps);
+    }
+    __syncthreads();
+    if (live) {
+      const float nw = norm_w[hc + col];
+      for (int tt = part; tt < n; tt += SP) {
+        const int64_t row = start + c0 + tt;
+        const float gv = E::load(g, row * g_stride + hc + col);
+        E::store(out, row * out_stride + hc + col, so[tt][col] * sinv[tt] * nw / (1.f + expf(-gv)));
+      }
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int ii = 0; ii < DS; ++ii) {
+      const int i = part * DS + ii;
+      if (i < K) st[(int64_t)i * K + col] = S[ii];
+    }
+  }
+}
+
+template <typename Tag>
+static int launch_delta(void* out, int64_t out_stride, const void* r, int64_t r_stride, const void* k, int64_t k_stride,
+                        const void* v, int64_t v_stride, const void* g, int64_t g_stride, const float* decay,
+                        const float* remove, const float* norm_w, float* state, int64_t state_stride, const SeqBatch& s,
+                        int H, int K, float eps, hipStream_t st) {
+  const dim3 grid((unsigned)s.B, (unsigned)H);
+#define SP_DELTA(KP)                                                                                                    \
+  delta_recurrence_kernel<Tag, KP><<<grid, (unsigned)((K * delta_split(KP) + 63) / 64 * 64), 0, st>>>(                  \
+      out, out_stride, r, r_stride, k, k_stride, v, v_stride, g, g_stride, decay, remove, norm_w, state, state_stride, s, H, K, \
+      eps)
+  if (K <= 16) SP_DELTA(16);
+  else if (K <= 32) SP_DELTA(32);
+  else if (K <= 64) SP_DELTA(64);
+  else if (K <= 128) SP_DELTA(128);
+  else if (K <= 256) SP_DELTA(256);
+  else return SP_ERR_UNSUPPORTED;
+#undef SP_DELTA
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+}  // namespace
+}  // namespace sp
+
+using namespace sp;
+
+extern "C" int sp_delta_gates(float* decay, float* remove, const void* p, int64_t p_stride, const float* w2t, const float* w0,
+                              const void* apre, int64_t a_stride, const float* a_bias, int64_t num_tokens, int channels,
+                              int rank, float rate, int dtype, void* stream) {
+  SP_CHECK_ARG(num_tokens >= 0 && channels > 0 && rank > 0 && rank <= 8192);
+  if (num_tokens == 0) return SP_OK;
+  SP_CHECK_ARG(decay && remove && p && w2t && w0 && apre && a_bias && p_stride >= rank && a_stride >= channels);
+  SP_DISPATCH_DTYPE(dtype, (delta_gates_kernel<Tag><<<dim3((unsigned)num_tokens), kBlock, rank * sizeof(float),
+                                                       (hipStream_t)stream>>>(decay, remove, p, p_stride, w2t, w0, apre,
+                                                                              a_stride, a_bias, channels, rank, rate)));
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+extern "C" int sp_delta_recurrence(void* out, int64_t out_stride, const void* r, int64_t r_stride, const void* k,
+                                   int64_t k_stride, const void* v, int64_t v_stride, const void* g, int64_t g_stride,
+                                   const float* decay, const float* remove, const float* norm_w, float* state,
+                                   int64_t state_stride, int heads, int head_dim, float eps, SP_SEQ_PARAMS, int dtype,
+                                   void* stream) {
+  SP_CHECK_ARG(batch_size >= 0 && heads > 0 && head_dim > 0);
+  if (batch_size == 0) return SP_OK;
+  SP_CHECK_ARG(out && r && k && v && g && decay && remove && norm_w && state && req_pool_indices && seq_lens);
+  SP_CHECK_ARG(!extend_seq_lens || (extend_prefix_lens && extend_start_loc));
+  SP_CHECK_ARG(state_stride >= (int64_t)heads * head_dim * head_dim);
+  const int64_t n = (int64_t)heads * head_dim;
+  SP_CHECK_ARG(r_stride >= n && k_stride >= n && v_stride >= n && g_stride >= n && out_stride >= n);
+  SEQ_BATCH(s);
+  SP_DISPATCH_DTYPE(dtype, return (launch_delta<Tag>(out, out_stride, r, r_stride, k, k_stride, v, v_stride, g, g_stride, decay,
+                                                     remove, norm_w, state, state_stride, s, heads, head_dim, eps,
+                                                     (hipStream_t)stream)));
+}

@@ -157,6 +157,44 @@ __global__ __launch_bounds__(kBlock) void silu_mul_scalar_kernel(void* __restric
   }
 }
 
+// ------------------------------------------------------------------- squared ReLU
+// out[t, j] = max(x[t, j], 0)^2 (the product in fp32, rounded once)
+template <typename Tag>
+__global__ __launch_bounds__(kBlock) void relu_square_vec_kernel(void* __restrict__ out, const void* __restrict__ x,
+                                                                  int64_t num_tokens, int d, int64_t x_stride,
+                                                                  int64_t o_stride) {
+  typedef Elem<Tag> E;
+  constexpr int V = E::kVec;
+  const int vec_per_row = d / V;
+  const int64_t total = num_tokens * vec_per_row;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += (int64_t)gridDim.x * kBlock) {
+    const int64_t t = i / vec_per_row;
+    const int v = (int)(i - t * vec_per_row);
+    float a[V], y[V];
+    unpack16<Tag>(ld16((const char*)x + t * x_stride * E::kBytes + (int64_t)v * 16), a);
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const float r = fmaxf(a[e], 0.f);
+      y[e] = __fmul_rn(r, r);
+    }
+    st16((char*)out + t * o_stride * E::kBytes + (int64_t)v * 16, pack16<Tag>(y));
+  }
+}
+
+template <typename Tag>
+__global__ __launch_bounds__(kBlock) void relu_square_scalar_kernel(void* __restrict__ out, const void* __restrict__ x,
+                                                                     int64_t num_tokens, int d, int64_t x_stride,
+                                                                     int64_t o_stride) {
+  typedef Elem<Tag> E;
+  const int64_t total = num_tokens * d;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += (int64_t)gridDim.x * kBlock) {
+    const int64_t t = i / d;
+    const int j = (int)(i - t * d);
+    const float r = fmaxf(E::load(x, t * x_stride + j), 0.f);
+    E::store(out, t * o_stride + j, __fmul_rn(r, r));
+  }
+}
+
 // ------------------------------------------------------------------- rotary (+ fused KV store)
 // nn/layers/rotary_embedding.py:23-49: o1 = x1*cos - x2*sin, o2 = x2*cos + x1*sin with every
 // product and the sum rounded to `dtype` (torch tensor arithmetic).  One workgroup per token.
@@ -507,6 +545,28 @@ extern "C" int sp_silu_and_mul(void* out, const void* x, int64_t num_tokens, int
   SP_CHECK_ARG(out && x);
   SP_DISPATCH_DTYPE(dtype, return (launch_silu<Tag>(out, x, num_tokens, d, x_stride, out_stride,
                                                      (hipStream_t)stream)));
+}
+
+template <typename Tag>
+static int launch_relu_square(void* out, const void* x, int64_t T, int d, int64_t xs, int64_t os, hipStream_t st) {
+  typedef Elem<Tag> E;
+  constexpr int V = E::kVec;
+  const bool vec = d % V == 0 && xs % V == 0 && os % V == 0 && aligned16(out) && aligned16(x);
+  const int64_t work = vec ? T * (d / V) : T * (int64_t)d;
+  int64_t blocks = (work + kBlock - 1) / kBlock;
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  if (vec) relu_square_vec_kernel<Tag><<<dim3((unsigned)blocks), kBlock, 0, st>>>(out, x, T, d, xs, os);
+  else relu_square_scalar_kernel<Tag><<<dim3((unsigned)blocks), kBlock, 0, st>>>(out, x, T, d, xs, os);
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+extern "C" int sp_relu_square(void* out, const void* x, int64_t num_tokens, int d, int64_t x_stride, int64_t out_stride,
+                              int dtype, void* stream) {
+  SP_CHECK_ARG(num_tokens >= 0 && d > 0);
+  if (num_tokens == 0) return SP_OK;
+  SP_CHECK_ARG(out && x && x_stride >= d && out_stride >= d);
+  SP_DISPATCH_DTYPE(dtype, return (launch_relu_square<Tag>(out, x, num_tokens, d, x_stride, out_stride, (hipStream_t)stream)));
 }
 
 template <typename Tag>

@@ -1,0 +1,148 @@
+// Gated linear attention whose forget gate also decides what is written (the HGRN2 recurrence).
+// Per head, with a query q [D], a value v [Dv] and a forget gate f [D] of a token, state S [D, Dv], all fp32:
+//   q = silu(qpre)                f = lower + (1 - lower) * sigmoid(fpre + f_bias)
+//   S' = diag(f) S + (1 - f) v^T          o = S'^T q
+//   out = o / rms_head(o) * norm_w         (norm_w [Dv], the same for every head)
+// There is no key: the row of S that belongs to query channel i takes in (1 - f_i) of the value.
+//
+// One workgroup per (request, head): a column of S (one value channel) lives in the registers of 1, 2 or 4 neighbouring
+// lanes; the request's tokens of this step are walked in order from the state the previous step left in the pool (zeros at
+// a sequence's first token), staged through LDS in passes of 16 tokens, the head norm as the pass's epilogue.
+#include "seq_batch.h"
+
+namespace sp {
+namespace {
+
+constexpr int hgrn_chunk(int DP) { return DP > 128 ? 8 : 16; }
+constexpr int hgrn_split(int DP) { return DP > 64 ? 4 : (DP > 32 ? 2 : 1); }
+
+template <typename Tag, int DP>
+__global__ void __launch_bounds__(256 * hgrn_split(DP))
+hgrn2_scan_kernel(void* out, int64_t out_stride, const void* qpre, int64_t q_stride, const void* fpre, int64_t f_stride,
+                  const void* v, int64_t v_stride, const float* f_bias, const float* lower, const float* norm_w, float* state,
+                  int64_t state_stride, SeqBatch s, int H, int D, int Dv, float eps) {
+  typedef Elem<Tag> E;
+  constexpr int kChunk = hgrn_chunk(DP), SP = hgrn_split(DP), DS = DP / SP, ROW = DP + 4 * SP;
+  __shared__ float sq[kChunk][ROW], sf[kChunk][ROW], sinv[kChunk];
+  extern __shared__ float so[];                         // [kChunk][Dv] numerators, then [kChunk][Dv] values
+  float* sv = so + (size_t)kChunk * Dv;
+  const int b = blockIdx.x, h = blockIdx.y, j = threadIdx.x;
+  const int nthreads = blockDim.x, wave = j >> 6, lane = j & 63, waves = nthreads >> 6;
+  const int col = j / SP, part = j % SP;
+  int64_t start, len, prefix;
+  seq_span(s, b, start, len, prefix);
+  if (len <= 0) return;
+  const bool live = col < Dv;
+  float* st = state + load_idx(s.req_pool_indices, b, s.idx64) * state_stride + (int64_t)h * D * Dv;
+  const bool held = prefix > 0;
+  float S[DS];
+#pragma unroll
+  for (int ii = 0; ii < DS; ++ii) {
+    const int i = part * DS + ii;
+    S[ii] = (live && i < D && held) ? st[(int64_t)i * Dv + col] : 0.f;
+  }
+  const int64_t colk = (int64_t)h * D, colv = (int64_t)h * Dv;
+  const int mine = part * (DS + 4);
+  for (int64_t c0 = 0; c0 < len; c0 += kChunk) {
+    const int n = (int)(len - c0 < kChunk ? len - c0 : kChunk);
+    __syncthreads();
+    for (int e = j; e < n * DP; e += nthreads) {
+      const int tt = e / DP, i = e % DP;
+      const int64_t row = start + c0 + tt;
+      const int at = i + 4 * (i / DS);
+      float qv = 0.f, fv = 0.f;
+      if (i < D) {
+        const float z = E::load(qpre, row * q_stride + colk + i);
+        qv = z / (1.f + expf(-z));
+        const float lo = lower[colk + i];
+        fv = lo + (1.f - lo) / (1.f + expf(-(E::load(fpre, row * f_stride + colk + i) + f_bias[colk + i])));
+      }
+      sq[tt][at] = qv;
+      sf[tt][at] = fv;
+    }
+    for (int e = j; e < n * Dv; e += nthreads) {
+      const int tt = e / Dv, c = e % Dv;
+      sv[tt * Dv + c] = E::load(v, (start + c0 + tt) * v_stride + colv + c);
+    }
+    __syncthreads();
+    for (int tt = 0; tt < n; ++tt) {
+      const float* pf = &sf[tt][mine];
+      const float* pq = &sq[tt][mine];
+      const float vj = live ? sv[tt * Dv + col] : 0.f;
+      float num = 0.f;
+#pragma unroll
+      for (int ii = 0; ii < DS; ++ii) {
+        const float f = pf[ii];
+        S[ii] = f * S[ii] + (1.f - f) * vj;
+        num += S[ii] * pq[ii];
+      }
+#pragma unroll
+      for (int off = 1; off < SP; off <<= 1) num += __shfl_xor(num, off, 64);
+      if (live && part == 0) so[tt * Dv + col] = num;
+    }
+    __syncthreads();
+    for (int tt = wave; tt < n; tt += waves) {
+      float ss = 0.f;
+      for (int i = lane; i < Dv; i += 64) ss += so[tt * Dv + i] * so[tt * Dv + i];
+      ss = wave_sum(ss);
+      if (lane == 0) sinv[tt] = 1.f / sqrtf(ss / (float)Dv + eps);
+    }
+    __syncthreads();
+    if (live) {
+      const float nw = norm_w[col];
+      for (int tt = part; tt < n; tt += SP)
+        E::store(out, (start + c0 + tt) * out_stride + colv + col, so[tt * Dv + col] * sinv[tt] * nw);
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int ii = 0; ii < DS; ++ii) {
+      const int i = part * DS + ii;
+      if (i < D) st[(int64_t)i * Dv + col] = S[ii];
+    }
+  }
+}
+
+template <typename Tag>
+static int launch_hgrn2(void* out, int64_t out_stride, const void* qpre, int64_t q_stride, const void* fpre, int64_t f_stride,
+                        const void* v, int64_t v_stride, const float* f_bias, const float* lower, const float* norm_w,
+                        float* state, int64_t state_stride, const SeqBatch& s, int H, int D, int Dv, float eps,
+                        hipStream_t st) {
+  const dim3 grid((unsigned)s.B, (unsigned)H);
+  if (Dv * (D > 64 ? 4 : (D > 32 ? 2 : 1)) > 1024) return SP_ERR_UNSUPPORTED;
+  // (register rows past D take f = 0 and q = 0: whatever they hold never reaches an output and is never stored)
+#define SP_HGRN(DP)                                                                                                     \
+  hgrn2_scan_kernel<Tag, DP><<<grid, (unsigned)((Dv * hgrn_split(DP) + 63) / 64 * 64),                                  \
+                               (size_t)hgrn_chunk(DP) * 2 * Dv * sizeof(float), st>>>(                                  \
+      out, out_stride, qpre, q_stride, fpre, f_stride, v, v_stride, f_bias, lower, norm_w, state, state_stride, s, H, D, Dv, eps)
+  if (D <= 16) SP_HGRN(16);
+  else if (D <= 32) SP_HGRN(32);
+  else if (D <= 64) SP_HGRN(64);
+  else if (D <= 128) SP_HGRN(128);
+  else if (D <= 256) SP_HGRN(256);
+  else return SP_ERR_UNSUPPORTED;
+#undef SP_HGRN
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+}  // namespace
+}  // namespace sp
+
+using namespace sp;
+
+extern "C" int sp_hgrn2_scan(void* out, int64_t out_stride, const void* qpre, int64_t q_stride, const void* fpre,
+                             int64_t f_stride, const void* v, int64_t v_stride, const float* f_bias, const float* lower,
+                             const float* norm_w, float* state, int64_t state_stride, int heads, int dim, int vdim, float eps,
+                             SP_SEQ_PARAMS, int dtype, void* stream) {
+  SP_CHECK_ARG(batch_size >= 0 && heads > 0 && dim > 0 && vdim > 0 && vdim <= 256);
+  if (batch_size == 0) return SP_OK;
+  SP_CHECK_ARG(out && qpre && fpre && v && f_bias && lower && norm_w && state && req_pool_indices && seq_lens);
+  SP_CHECK_ARG(!extend_seq_lens || (extend_prefix_lens && extend_start_loc));
+  const int64_t nk = (int64_t)heads * dim, nv = (int64_t)heads * vdim;
+  SP_CHECK_ARG(q_stride >= nk && f_stride >= nk && v_stride >= nv && out_stride >= nv && state_stride >= nk * vdim);
+  SEQ_BATCH(s);
+  SP_DISPATCH_DTYPE(dtype, return (launch_hgrn2<Tag>(out, out_stride, qpre, q_stride, fpre, f_stride, v, v_stride, f_bias, lower,
+                                                     norm_w, state, state_stride, s, heads, dim, vdim, eps,
+                                                     (hipStream_t)stream)));
+}

@@ -413,6 +413,20 @@ __global__ __launch_bounds__(kSampThreads) void softmax_temperature_kernel(float
   for (int i = tid; i < vocab; i += kSampThreads) row[i] = expf(row[i] / t - mx) * inv;
 }
 
+// out[r, j] = cap * tanh(z[r, j] * scale / cap)  (cap <= 0: z * scale), fp32 whatever the logits' element type
+template <typename Tag>
+__global__ void scale_softcap_kernel(float* out, int64_t out_stride, const void* z, int64_t z_stride, int64_t rows, int n,
+                                     float scale, float cap) {
+  typedef Elem<Tag> E;
+  const int64_t total = rows * n;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = i / n;
+    const int j = (int)(i - r * n);
+    const float v = E::load(z, r * z_stride + j) * scale;
+    out[r * out_stride + j] = cap > 0.f ? cap * tanhf(v / cap) : v;
+  }
+}
+
 }  // namespace sp
 
 extern "C" int sp_argmax(const void* logits, int64_t row_stride, int batch_size, int vocab, int64_t* out_ids,
@@ -481,6 +495,19 @@ extern "C" int sp_top_k_top_p_min_p_renorm(const float* probs, int64_t row_strid
   SP_CHECK_ARG(probs && out && row_stride >= vocab && out_stride >= vocab);
   sp::SelectArgs a{probs, row_stride, top_ks, top_ps, min_ps, nullptr, vocab, nullptr, out, out_stride, keep_count};
   sp::select_kernel<false><<<dim3(batch_size), sp::kSampThreads, 0, (hipStream_t)stream>>>(a);
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+extern "C" int sp_scale_softcap(float* out, int64_t out_stride, const void* logits, int64_t row_stride, int64_t rows, int n,
+                                float scale, float cap, int dtype, void* stream) {
+  SP_CHECK_ARG(rows >= 0 && n > 0);
+  if (rows == 0) return SP_OK;
+  SP_CHECK_ARG(out && logits && out_stride >= n && row_stride >= n);
+  int64_t blocks = (rows * n + 255) / 256;
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  SP_DISPATCH_DTYPE(dtype, (sp::scale_softcap_kernel<Tag><<<dim3((unsigned)blocks), 256, 0, (hipStream_t)stream>>>(
+                               out, out_stride, logits, row_stride, rows, n, scale, cap)));
   SP_LAUNCH_CHECK();
   return SP_OK;
 }

@@ -6,6 +6,9 @@
 //   saved h               state[slot] = h[the request's last row of this step]             (fp32, a launch of its own:
 //                                                                                           every reader has finished)
 //   sum                   x[t] += a[t] + b[t] + c[t]                                       (fp32; b, c optional)
+// and of sequential-sublayer models that gate and norm a sublayer's RESULT before it joins the stream:
+//   gated normed sum      y = a  or  (N(a) wa + N(b) wb) / 2;   y *= sigmoid(gate + gate_bias);   x += N(y) w;
+//                         x += extra;   next = N(x) w_next      (N = division by the row's root mean square)
 // All arithmetic is fp32; h and hs are rounded once, to the projections' element type.
 #include "seq_batch.h"
 
@@ -94,6 +97,56 @@ __global__ void stream_add_kernel(float* x, int64_t x_stride, const void* a, int
   }
 }
 
+
+// one workgroup per row; the row's y, then its new x, wait in LDS between the reductions (each thread reads back only what
+// it wrote itself, so the reductions' barriers are the only ones)
+template <typename Tag>
+__global__ void __launch_bounds__(kBlock)
+gated_add_norm_kernel(float* x, int64_t x_stride, const void* a, int64_t a_stride, const float* wa, const void* b,
+                      int64_t b_stride, const float* wb, const void* gate, int64_t gate_stride, const float* gate_bias,
+                      const float* weight, const float* extra, int64_t extra_stride, void* out_next, int64_t next_stride,
+                      const float* next_weight, int width, float eps) {
+  typedef Elem<Tag> E;
+  extern __shared__ float rowbuf[];
+  __shared__ float red[kBlock / 64];
+  const int64_t t = blockIdx.x;
+  float ia = 1.f, ib = 0.f;
+  if (b) {
+    float sa = 0.f, sb = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+      const float u = E::load(a, t * a_stride + i), v = E::load(b, t * b_stride + i);
+      sa += u * u;
+      sb += v * v;
+    }
+    sa = block_sum(sa, red);
+    sb = block_sum(sb, red);
+    ia = 1.f / sqrtf(sa / (float)width + eps);
+    ib = 1.f / sqrtf(sb / (float)width + eps);
+  }
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float y = E::load(a, t * a_stride + i);
+    if (b) y = 0.5f * (y * ia * wa[i] + E::load(b, t * b_stride + i) * ib * wb[i]);
+    if (gate) y /= 1.f + expf(-(E::load(gate, t * gate_stride + i) + (gate_bias ? gate_bias[i] : 0.f)));
+    rowbuf[i] = y;
+    ss += y * y;
+  }
+  ss = block_sum(ss, red);
+  const float inv = 1.f / sqrtf(ss / (float)width + eps);
+  float sx = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float v = x[t * x_stride + i] + rowbuf[i] * inv * weight[i];
+    if (extra) v += extra[t * extra_stride + i];
+    x[t * x_stride + i] = v;
+    rowbuf[i] = v;
+    sx += v * v;
+  }
+  if (!out_next) return;
+  sx = block_sum(sx, red);
+  const float invx = 1.f / sqrtf(sx / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += blockDim.x) E::store(out_next, t * next_stride + i, rowbuf[i] * invx * next_weight[i]);
+}
+
 }  // namespace
 }  // namespace sp
 
@@ -148,6 +201,26 @@ extern "C" int sp_stream_add(float* x, int64_t x_stride, const void* a, int64_t 
   SP_CHECK_ARG(x && a && x_stride >= width && a_stride >= width && (!b || b_stride >= width) && (!c || c_stride >= width));
   SP_DISPATCH_DTYPE(dtype, (stream_add_kernel<Tag><<<dim3((unsigned)num_tokens), kBlock, 0, (hipStream_t)stream>>>(
                                x, x_stride, a, a_stride, b, b_stride, c, c_stride, width)));
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+extern "C" int sp_gated_add_norm(float* x, int64_t x_stride, const void* a, int64_t a_stride, const float* wa, const void* b,
+                                 int64_t b_stride, const float* wb, const void* gate, int64_t gate_stride,
+                                 const float* gate_bias, const float* weight, const float* extra, int64_t extra_stride,
+                                 void* out_next, int64_t next_stride, const float* next_weight, int64_t num_tokens, int width,
+                                 float eps, int dtype, void* stream) {
+  SP_CHECK_ARG(num_tokens >= 0 && width > 0 && width <= 15360);
+  if (num_tokens == 0) return SP_OK;
+  SP_CHECK_ARG(x && a && weight && x_stride >= width && a_stride >= width);
+  SP_CHECK_ARG(!b || (wa && wb && b_stride >= width));
+  SP_CHECK_ARG(!gate || gate_stride >= width);
+  SP_CHECK_ARG(!extra || extra_stride >= width);
+  SP_CHECK_ARG(!out_next || (next_weight && next_stride >= width));
+  SP_DISPATCH_DTYPE(dtype, (gated_add_norm_kernel<Tag><<<dim3((unsigned)num_tokens), kBlock, (size_t)width * sizeof(float),
+                                                          (hipStream_t)stream>>>(
+                               x, x_stride, a, a_stride, wa, b, b_stride, wb, gate, gate_stride, gate_bias, weight, extra,
+                               extra_stride, out_next, next_stride, next_weight, width, eps)));
   SP_LAUNCH_CHECK();
   return SP_OK;
 }

@@ -10,46 +10,63 @@
 // pooled key/value of block b lives in a second pair of buffers at the slot of the block's LAST token, written by the
 // step that brings this token, so the pooled rows need no allocator of their own and are freed with the token.
 //
-// Rotation: "rotate half" - coordinate i < dims/2 pairs with i + dims/2, angle = position * freq[i] in fp32, cos and
-// sin times mag; coordinates from dims on pass.  Scores, softmax and the weighted sum are fp32.
+// Rotation: "rotate half" - coordinate i < dims/2 pairs with i + dims/2 - or, with `adjacent`, coordinate 2i with 2i + 1;
+// angle = position * freq[i] in fp32, cos and sin times mag; coordinates from dims on pass.  Optional fp32 biases join q, k
+// and v before the rotation; the per-head norm of the values can be switched off.  Scores, softmax and the weighted sum are
+// fp32.  With `sinks` (one fp32 number per query head) the softmax's denominator holds one more term exp(sink): a key that
+// is seen by every query, is not scaled and has no value.
 #include "seq_batch.h"
 
 namespace sp {
 namespace {
 
-// q rotated in place; k rotated and v normed into the pool rows loc[t]
+// q rotated in place; k rotated and v (normed per head unless norm_v is 0) into the pool rows loc[t]
 template <typename Tag>
 __global__ void __launch_bounds__(kBlock)
 qkv_rotary_store_kernel(void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
                         void* kpool, int64_t kp_stride, void* vpool, int64_t vp_stride, const int64_t* positions,
-                        const int64_t* loc, const float* freq, float mag, int H, int G, int D, int Dv, int dims, float eps) {
+                        const int64_t* loc, const float* freq, float mag, const float* qb, const float* kb, const float* vb,
+                        int H, int G, int D, int Dv, int dims, int adjacent, int norm_v, float eps) {
   typedef Elem<Tag> E;
   const int64_t t = blockIdx.x;
   const float pos = (float)positions[t];
   const int half = dims / 2;
   const int64_t slot = loc[t];
+  const int second = adjacent ? 1 : half, step = adjacent ? 2 : 1;      // a pair is (i * step, i * step + second)
   for (int e = threadIdx.x; e < H * half; e += blockDim.x) {
     const int h = e / half, i = e % half;
     const float a = pos * freq[i];
     const float c = cosf(a) * mag, sn = sinf(a) * mag;
-    const int64_t at = t * q_stride + (int64_t)h * D + i;
-    const float u = E::load(q, at), w = E::load(q, at + half);
+    const int col = h * D + i * step;
+    const int64_t at = t * q_stride + col;
+    const float u = E::load(q, at) + (qb ? qb[col] : 0.f), w = E::load(q, at + second) + (qb ? qb[col + second] : 0.f);
     E::store(q, at, u * c - w * sn);
-    E::store(q, at + half, w * c + u * sn);
+    E::store(q, at + second, w * c + u * sn);
   }
   for (int e = threadIdx.x; e < G * half; e += blockDim.x) {
     const int g = e / half, i = e % half;
     const float a = pos * freq[i];
     const float c = cosf(a) * mag, sn = sinf(a) * mag;
-    const int64_t at = t * k_stride + (int64_t)g * D + i, to = slot * kp_stride + (int64_t)g * D + i;
-    const float u = E::load(k, at), w = E::load(k, at + half);
+    const int col = g * D + i * step;
+    const int64_t at = t * k_stride + col, to = slot * kp_stride + col;
+    const float u = E::load(k, at) + (kb ? kb[col] : 0.f), w = E::load(k, at + second) + (kb ? kb[col + second] : 0.f);
     E::store(kpool, to, u * c - w * sn);
-    E::store(kpool, to + half, w * c + u * sn);
+    E::store(kpool, to + second, w * c + u * sn);
   }
   const int rest = D - dims;
+  if (qb)
+    for (int e = threadIdx.x; e < H * rest; e += blockDim.x) {
+      const int col = (e / rest) * D + dims + e % rest;
+      E::store(q, t * q_stride + col, E::load(q, t * q_stride + col) + qb[col]);
+    }
   for (int e = threadIdx.x; e < G * rest; e += blockDim.x) {
-    const int g = e / rest, i = dims + e % rest;
-    E::store(kpool, slot * kp_stride + (int64_t)g * D + i, E::load(k, t * k_stride + (int64_t)g * D + i));
+    const int col = (e / rest) * D + dims + e % rest;
+    E::store(kpool, slot * kp_stride + col, E::load(k, t * k_stride + col) + (kb ? kb[col] : 0.f));
+  }
+  if (!norm_v) {
+    for (int e = threadIdx.x; e < G * Dv; e += blockDim.x)
+      E::store(vpool, slot * vp_stride + e, E::load(v, t * v_stride + e) + (vb ? vb[e] : 0.f));
+    return;
   }
   // value heads: one wave each
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, waves = blockDim.x >> 6;
@@ -57,12 +74,12 @@ qkv_rotary_store_kernel(void* q, int64_t q_stride, const void* k, int64_t k_stri
     const int64_t at = t * v_stride + (int64_t)g * Dv, to = slot * vp_stride + (int64_t)g * Dv;
     float ss = 0.f;
     for (int i = lane; i < Dv; i += 64) {
-      const float x = E::load(v, at + i);
+      const float x = E::load(v, at + i) + (vb ? vb[g * Dv + i] : 0.f);
       ss += x * x;
     }
     ss = wave_sum(ss);
     const float inv = 1.f / sqrtf(ss / (float)Dv + eps);
-    for (int i = lane; i < Dv; i += 64) E::store(vpool, to + i, E::load(v, at + i) * inv);
+    for (int i = lane; i < Dv; i += 64) E::store(vpool, to + i, (E::load(v, at + i) + (vb ? vb[g * Dv + i] : 0.f)) * inv);
   }
 }
 
@@ -122,7 +139,7 @@ __global__ void __launch_bounds__(1024)
 window_attention_kernel(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kpool, const void* vpool,
                         const void* kpooled, const void* vpooled, int64_t kp_stride, int64_t vp_stride,
                         const int32_t* req_to_token, int64_t table_stride, SeqBatch s, int H, int G, int D, int Dv,
-                        int64_t size, int P, float scale) {
+                        int64_t size, int P, float scale, const float* sinks) {
   typedef Elem<Tag> E;
   extern __shared__ float smem[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, NW = blockDim.x >> 6;
@@ -219,6 +236,10 @@ window_attention_kernel(void* out, int64_t out_stride, const void* q, int64_t q_
   float M = sml[0];                                                         // wave 0 always holds a key: M is finite
   for (int w = 1; w < NW; ++w) M = fmaxf(M, sml[w]);
   float den = 0.f;
+  if (sinks) {                                                              // one more term of the denominator
+    M = fmaxf(M, sinks[h]);
+    den = expf(sinks[h] - M);
+  }
   for (int w = 0; w < NW; ++w) den += sml[NW + w] * expf(sml[w] - M);       // a wave without keys: exp(-inf) = 0
   const float inv = 1.f / den;
   for (int c = threadIdx.x; c < Dv; c += blockDim.x) {
@@ -261,7 +282,7 @@ __global__ void __launch_bounds__(256)
 window_attention_mfma_kernel(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kpool,
                              const void* vpool, const void* kpooled, const void* vpooled, int64_t kp_stride, int64_t vp_stride,
                              const int32_t* req_to_token, int64_t table_stride, SeqBatch s, int H, int G, int64_t size, int P,
-                             float scale) {
+                             float scale, const float* sinks) {
   constexpr int D = 32 * DS, Dv = 16 * DT;
   __shared__ uint16_t vt[Dv][kVtRow];
   __shared__ int32_t sslot[64];
@@ -402,7 +423,11 @@ window_attention_mfma_kernel(void* out, int64_t out_stride, const void* q, int64
       }
     }
     if (work && qvalid) {
-      const float inv = 1.f / l;
+      float inv = 1.f / l;
+      if (sinks) {                                     // (a valid query has seen itself: m is finite)
+        const float sk = sinks[hq], m2 = fmaxf(m, sk), keep = expf(m - m2);
+        inv = keep / (l * keep + expf(sk - m2));
+      }
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
         float f[8] = {oacc[dt][0] * inv, oacc[dt][1] * inv, oacc[dt][2] * inv, oacc[dt][3] * inv, 0.f, 0.f, 0.f, 0.f};
@@ -421,8 +446,9 @@ using namespace sp;
 extern "C" int sp_qkv_rotary_store(void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v,
                                    int64_t v_stride, void* kpool, int64_t kp_stride, void* vpool, int64_t vp_stride,
                                    const int64_t* positions, const int64_t* loc, const float* freq, float mag,
-                                   int64_t num_tokens, int heads, int kv_heads, int dim, int vdim, int rot_dims, float eps,
-                                   int dtype, void* stream) {
+                                   const float* q_bias, const float* k_bias, const float* v_bias, int64_t num_tokens,
+                                   int heads, int kv_heads, int dim, int vdim, int rot_dims, int adjacent, int norm_values,
+                                   float eps, int dtype, void* stream) {
   SP_CHECK_ARG(num_tokens >= 0 && heads > 0 && kv_heads > 0 && dim > 0 && vdim > 0);
   SP_CHECK_ARG(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= dim);
   if (num_tokens == 0) return SP_OK;
@@ -431,7 +457,8 @@ extern "C" int sp_qkv_rotary_store(void* q, int64_t q_stride, const void* k, int
   SP_CHECK_ARG(kp_stride >= (int64_t)kv_heads * dim && vp_stride >= (int64_t)kv_heads * vdim);
   SP_DISPATCH_DTYPE(dtype, (qkv_rotary_store_kernel<Tag><<<dim3((unsigned)num_tokens), kBlock, 0, (hipStream_t)stream>>>(
                                q, q_stride, k, k_stride, v, v_stride, kpool, kp_stride, vpool, vp_stride, positions, loc,
-                               freq, mag, heads, kv_heads, dim, vdim, rot_dims, eps)));
+                               freq, mag, q_bias, k_bias, v_bias, heads, kv_heads, dim, vdim, rot_dims, adjacent, norm_values,
+                               eps)));
   SP_LAUNCH_CHECK();
   return SP_OK;
 }
@@ -457,7 +484,7 @@ extern "C" int sp_window_attention(void* out, int64_t out_stride, const void* q,
                                    const void* vpool, const void* kpooled, const void* vpooled, int64_t kp_stride,
                                    int64_t vp_stride, const int32_t* req_to_token, int64_t table_stride,
                                    int64_t num_tokens, int heads, int kv_heads, int dim, int vdim, int64_t window, int block,
-                                   float scale, int matrix, SP_SEQ_PARAMS, int dtype, void* stream) {
+                                   float scale, const float* sinks, int matrix, SP_SEQ_PARAMS, int dtype, void* stream) {
   SP_CHECK_ARG(num_tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0);
   if (num_tokens == 0) return SP_OK;
   SP_CHECK_ARG(out && q && kpool && vpool && req_to_token && req_pool_indices && seq_lens);
@@ -480,7 +507,7 @@ extern "C" int sp_window_attention(void* out, int64_t out_stride, const void* q,
 #define SP_WM(T, DS, DT)                                                                                                 \
   window_attention_mfma_kernel<T, DS, DT><<<mgrid, 256, 0, (hipStream_t)stream>>>(                                         \
       out, out_stride, q, q_stride, kpool, vpool, kpooled, vpooled, kp_stride, vp_stride, req_to_token, table_stride, s, heads, \
-      kv_heads, window, block, scale)
+      kv_heads, window, block, scale, sinks)
 #define SP_WM_SHAPES(T)                                   \
   do {                                                    \
     if (dim == 64 && vdim == 64) SP_WM(T, 2, 4);          \
@@ -502,7 +529,7 @@ extern "C" int sp_window_attention(void* out, int64_t out_stride, const void* q,
 #define SP_WA(V)                                                                                                       \
   SP_DISPATCH_DTYPE(dtype, (window_attention_kernel<Tag, V><<<grid, 64 * nw, lds, (hipStream_t)stream>>>(               \
                                out, out_stride, q, q_stride, kpool, vpool, kpooled, vpooled, kp_stride, vp_stride,      \
-                               req_to_token, table_stride, s, heads, kv_heads, dim, vdim, window, block, scale)))
+                               req_to_token, table_stride, s, heads, kv_heads, dim, vdim, window, block, scale, sinks)))
   if (vec) SP_WA(true);
   else SP_WA(false);
 #undef SP_WA

@@ -30,6 +30,13 @@ class RMSNorm(CustomOp):
         return _native.rmsnorm(x, self.weight.data, self.variance_epsilon)
 
 
+class ReluSquare(CustomOp):
+    """max(x, 0)^2, element by element"""
+
+    def forward_hip(self, x: torch.Tensor) -> torch.Tensor:
+        return _native.relu_square(x)
+
+
 class SiluAndMul(CustomOp):
     """activation.py:21-31: silu(x[..., :d]) * x[..., d:]."""
 
@@ -264,16 +271,40 @@ def yarn_blend(dims: int, base: float, factor: float, original: float, fast: flo
     return f / factor * ramp + f * (1 - ramp)
 
 
+def wavelength_blend(dims: int, base: float, factor: float, original: float, low: float, high: float) -> torch.Tensor:
+    """Rotary frequencies f_i = base^(-2i/dims), i < dims/2, rescaled by their wavelength 2 pi / f (the rule of Llama 3.1's
+    context extension): a wavelength below original / high keeps its frequency, one above original / low has it divided by
+    ``factor``, and between the two the frequency is (1 - s) f / factor + s f with s = (original / wavelength - low) /
+    (high - low).  float64."""
+    out = []
+    for i in range(dims // 2):
+        f = base ** (-2.0 * i / dims)
+        wavelength = 2 * math.pi / f
+        if wavelength > original / low:
+            f = f / factor
+        elif wavelength >= original / high and high != low:
+            s = (original / wavelength - low) / (high - low)
+            f = (1 - s) * f / factor + s * f
+        out.append(f)
+    return torch.tensor(out, dtype=torch.float64)
+
+
 class AngleRotary(nn.Module):
     """Rotary embedding without a table: fp32 frequencies, the angle position * f_i formed in fp32 inside the kernel,
     interleaved pairs (2i, 2i+1) of the first ``dims`` coordinates, cos and sin scaled by ``magnitude``.  ``scaling`` =
-    {factor, original, fast, slow} blends the frequencies (yarn_blend) and sets magnitude = 0.1 ln(factor) + 1."""
+    {factor, original, fast, slow} blends the frequencies (yarn_blend) and sets magnitude = 0.1 ln(factor) + 1;
+    ``scaling`` = {factor, original, low, high} rescales them by wavelength (wavelength_blend), magnitude 1."""
+    adjacent_pairs = True
 
     def __init__(self, dims: int, base: float, scaling: Optional[Dict[str, Any]] = None) -> None:
         super().__init__()
         if dims % 2:
             raise ValueError("rotary dims must be even")
-        if scaling:
+        if scaling and "low" in scaling:
+            freq = wavelength_blend(dims, base, float(scaling["factor"]), float(scaling["original"]), float(scaling["low"]),
+                                    float(scaling["high"]))
+            self.magnitude = 1.0
+        elif scaling:
             freq = yarn_blend(dims, base, scaling["factor"], scaling["original"], scaling["fast"], scaling["slow"])
             self.magnitude = 0.1 * math.log(scaling["factor"]) + 1.0
         else:
@@ -290,6 +321,7 @@ class AngleRotary(nn.Module):
 class HalfAngleRotary(AngleRotary):
     """The same fp32 frequencies and magnitude, for the "rotate half" pairing: coordinate i < dims / 2 pairs with
     i + dims / 2.  Applied by the fused rotation + cache store (_native.qkv_rotary_store), not by a call of its own."""
+    adjacent_pairs = False
 
     def forward(self, positions: torch.Tensor, x: torch.Tensor, offset: int = 0) -> None:
         raise NotImplementedError("the half-pair rotation runs inside _native.qkv_rotary_store")
@@ -330,3 +362,47 @@ class GluFF(nn.Module):
         gu = _native.linear(h, self.gate_up)
         y = _native.silu_and_mul(gu) if self.act == "silu" else _native.moe_glu(gu.contiguous(), self.limit, self.alpha)
         return _native.linear(y, self.down)
+
+
+class GatedAddNorm(nn.Module):
+    """How a sublayer's result y joins an fp32 residual stream when it is gated and normed first:
+    x += N(y * sigmoid(gate + bias)) * weight, N = division by the row's root mean square.  The gate's pre-activation is a
+    product of the sublayer's own input, so its rows ride in the sublayer's input projection and arrive here as ``gate``.
+    ``y`` may be two branches (a, b), each normed over the row with its own weight and averaged: y = (N(a) wa + N(b) wb) / 2.
+    ``extra`` (fp32) is added to the stream afterwards; with ``next_weight`` the call also returns N(x) * next_weight in the
+    projections' dtype - the next sublayer's input - from the same pass over the row."""
+
+    def __init__(self, width: int, eps: float = 1e-6, gated: bool = True, branches: int = 1) -> None:
+        super().__init__()
+        f32 = dict(dtype=torch.float32)
+        self.weight = nn.Parameter(torch.ones(width, **f32), requires_grad=False)
+        self.gate_bias = nn.Parameter(torch.zeros(width, **f32), requires_grad=False) if gated else None
+        self.branch_weight = nn.Parameter(torch.ones(2, width, **f32), requires_grad=False) if branches == 2 else None
+        self.variance_epsilon = eps
+
+    def forward(self, x: torch.Tensor, y, gate: Optional[torch.Tensor] = None, extra: Optional[torch.Tensor] = None,
+                next_weight: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+        a, b = y if isinstance(y, (tuple, list)) else (y, None)
+        if (b is not None) != (self.branch_weight is not None):
+            raise RuntimeError("GatedAddNorm: built for another number of branches")
+        wa, wb = (self.branch_weight.data[0], self.branch_weight.data[1]) if b is not None else (None, None)
+        return _native.gated_add_norm(x, a, self.weight.data, self.variance_epsilon, gate=gate,
+                                      gate_bias=None if self.gate_bias is None else self.gate_bias.data, b=b, wa=wa, wb=wb,
+                                      extra=extra, next_weight=next_weight)
+
+
+class ReluSquareFF(nn.Module):
+    """Feed-forward W_down relu(W_up h)^2.  ``extra_rows`` further rows of the up projection are not activated: their
+    outputs come back beside the result (a layer's gate on this sublayer reads the same h, so it rides in this product)."""
+
+    def __init__(self, width: int, ff: int, extra_rows: int = 0, dtype=None):
+        super().__init__()
+        self.ff, self.extra_rows = ff, extra_rows
+        self.up = nn.Parameter(torch.empty(ff + extra_rows, width, dtype=dtype), requires_grad=False)
+        self.down = nn.Parameter(torch.empty(width, ff, dtype=dtype), requires_grad=False)
+        self.act = ReluSquare()
+
+    def forward(self, h: torch.Tensor):
+        a = _native.linear(h, self.up)
+        y = _native.linear(self.act(a[:, :self.ff]), self.down)
+        return (y, a[:, self.ff:]) if self.extra_rows else y

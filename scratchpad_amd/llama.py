@@ -259,6 +259,15 @@ class LogitsProcessor(nn.Module):
         super().__init__()
         self.config = config
         self.do_tensor_parallel_all_gather = get_tensor_model_parallel_world_size() > 1
+        # logits * logit_scale, then cap * tanh(. / cap): fp32, after the head's product (configurations without them: off)
+        self.logit_scale = float(getattr(config, "logit_scale", 1.0) or 1.0)
+        self.logit_softcap = float(getattr(config, "final_logit_softcapping", 0.0) or 0.0)
+
+    def _shape_logits(self, logits):
+        """the configured scale and soft cap on the head's output (fp32 from there on); nothing configured: as it is"""
+        if self.logit_scale == 1.0 and self.logit_softcap <= 0.0:
+            return logits
+        return _native.scale_softcap(logits, self.logit_scale, self.logit_softcap)
 
     @staticmethod
     def input_logprob_plan(extend_seq_lens_cpu, extend_logprob_start_lens_cpu):
@@ -281,7 +290,7 @@ class LogitsProcessor(nn.Module):
 
     def _full_logits(self, states, lm_head):
         """_get_logits, logits_processor.py:344-376: matmul, all-gather over the TP group, cut the padding, fp32"""
-        logits = _native.linear(states.to(lm_head.weight.dtype), lm_head.weight)
+        logits = self._shape_logits(_native.linear(states.to(lm_head.weight.dtype), lm_head.weight))
         if self.do_tensor_parallel_all_gather:
             logits = tensor_model_parallel_all_gather(logits)
         return logits[:, : self.config.vocab_size].float()
@@ -298,7 +307,7 @@ class LogitsProcessor(nn.Module):
             else:
                 last_index = torch.cumsum(fb.extend_seq_lens, dim=0) - 1
                 pruned = hidden_states[last_index]
-            logits = _native.linear(pruned.to(lm_head.weight.dtype), lm_head.weight)
+            logits = self._shape_logits(_native.linear(pruned.to(lm_head.weight.dtype), lm_head.weight))
             return LogitsProcessorOutput(shard_logits=logits, vocab_size=self.config.vocab_size,
                                          shard_offset=getattr(lm_head, "vocab_start_index", 0))
         spans, sample_idx, input_idx, pruned_lens = self.input_logprob_plan(fb.extend_seq_lens_cpu,

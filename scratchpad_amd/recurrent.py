@@ -1,5 +1,7 @@
 """Recurrent token mixers over per-request state in the RecurrentStatePool: WKVMixer (RWKV-style time mixing, csrc/wkv.hip),
-Mamba2Mixer (state-space duality form, csrc/ssm.hip) and MLSTMMixer (matrix memory with exponential gating, csrc/mlstm.hip).
+Mamba2Mixer (state-space duality form, csrc/ssm.hip), MLSTMMixer (matrix memory with exponential gating, csrc/mlstm.hip),
+GeneralDeltaMixer (generalized delta rule, csrc/delta_rule.hip) and HGRN2Mixer (linear attention whose forget gate also
+writes, csrc/hgrn.hip).
 
 WKVMixer:
 
@@ -9,6 +11,9 @@ Per token t with layer input h[t] (the fp32 residual stream) and h[t-1] (zeros a
   o = (S + diag(u) k v^T)^T r ;  S <- diag(decay) S + k v^T     per head, S in fp32 in the RecurrentStatePool
   out = W_o ((o / rms_head(o)) * norm * gate)
 The four projections that feed the recurrence run as ONE batched matrix product over their stacked weights."""
+import math
+from typing import Optional
+
 import torch
 from torch import nn
 
@@ -124,3 +129,82 @@ class MLSTMMixer(nn.Module):
                                self.norm.data, states.state(L, "S"), states.state(L, "n"), states.state(L, "m"), seq,
                                self.heads, self.dim, self.vdim, self.cap, self.eps)
         return _native.linear(o, self.o)
+
+
+class GeneralDeltaMixer(nn.Module):
+    """Generalized delta rule.  r, k, v [heads, dim] and an output gate g are projections of h; per head and key channel a
+    decay w = exp(-rate sigmoid(W_w2 tanh(W_w1 h) + w0)) and a removal rate a = sigmoid(W_a h + a_bias); with the unit key
+    u = k / sqrt(|k|^2 + 1e-6), in fp32:
+        S <- diag(w) S - (a * u)(u^T S) + k v^T   (both first terms read the previous S),   o = S^T r,
+    out = W_o (o / rms_head(o) * norm * sigmoid(g)).  r, k, v, g, the removal rate's and the decay's first projection
+    come from ONE product (rows [r | k | v | g | a | w1 | extra]); ``extra_rows`` further rows of that product are handed
+    back untouched (a layer's gate on this sublayer reads the same h).  The decay's second projection is fp32."""
+
+    def __init__(self, width: int, heads: int, dim: int, decay_rank: int, eps: float, rate: float = math.exp(-0.5),
+                 layer_id: Optional[int] = None, extra_rows: int = 0, dtype=None):
+        super().__init__()
+        self.width, self.heads, self.dim, self.rank, self.eps, self.rate = width, heads, dim, decay_rank, eps, rate
+        self.layer_id, self.extra_rows = layer_id, extra_rows
+        n = heads * dim
+        f32 = dict(dtype=torch.float32)
+        self.in_proj = nn.Parameter(torch.empty(5 * n + decay_rank + extra_rows, width, dtype=dtype), requires_grad=False)
+        self.w2t = nn.Parameter(torch.zeros(decay_rank, n, **f32), requires_grad=False)      # W_w2 transposed, fp32
+        self.w0 = nn.Parameter(torch.zeros(n, **f32), requires_grad=False)
+        self.a_bias = nn.Parameter(torch.zeros(n, **f32), requires_grad=False)
+        self.norm = nn.Parameter(torch.ones(n, **f32), requires_grad=False)
+        self.o = nn.Parameter(torch.empty(width, n, dtype=dtype), requires_grad=False)
+
+    @staticmethod
+    def state_shapes(heads: int, dim: int):
+        return {"S": (heads, dim, dim)}
+
+    def forward(self, h: torch.Tensor, forward_batch: ForwardBatch, state_id: Optional[int] = None):
+        """h [T, W] in the projections' dtype -> the mixer's output [T, W] (and the extra rows' outputs [T, extra_rows]).
+        ``state_id``: the state to use instead of ``layer_id`` (a layer that runs several times on the same weights keeps one
+        state per run)."""
+        seq, states = forward_batch.attn_backend.seq, forward_batch.state_pool
+        n = self.heads * self.dim
+        a = _native.linear(h, self.in_proj)
+        decay, remove = _native.delta_gates(a[:, 5 * n:5 * n + self.rank], self.w2t.data, self.w0.data, a[:, 4 * n:5 * n],
+                                            self.a_bias.data, self.rate)
+        S = states.state(self.layer_id if state_id is None else state_id, "S")
+        o = _native.delta_recurrence(a[:, :n], a[:, n:2 * n], a[:, 2 * n:3 * n], a[:, 3 * n:4 * n], decay, remove,
+                                     self.norm.data, S, seq, self.heads, self.dim, self.eps)
+        y = _native.linear(o, self.o)
+        return (y, a[:, 5 * n + self.rank:]) if self.extra_rows else y
+
+
+class HGRN2Mixer(nn.Module):
+    """Linear attention in which the forget gate also decides what is written.  q = silu(W_q h) [heads, dim], v = W_v h
+    [heads, vdim], f = lower + (1 - lower) sigmoid(W_f h + f_bias) per head and query channel; in fp32
+        S <- diag(f) S + (1 - f) v^T,   o = S^T q          (S [dim, vdim]; no key, no other scale)
+    out = W_o (o / rms_head(o) * norm), norm [vdim] shared by the heads.  The rows [q | f | v] of the input projection may
+    be part of a larger product of the caller (``scan`` takes the three views); ``forward`` runs the mixer's own."""
+
+    def __init__(self, width: int, heads: int, dim: int, vdim: int, eps: float, layer_id: Optional[int] = None,
+                 own_input: bool = True, dtype=None):
+        super().__init__()
+        self.heads, self.dim, self.vdim, self.eps, self.layer_id = heads, dim, vdim, eps, layer_id
+        f32 = dict(dtype=torch.float32)
+        self.in_rows = 2 * heads * dim + heads * vdim
+        self.in_proj = nn.Parameter(torch.empty(self.in_rows, width, dtype=dtype), requires_grad=False) if own_input else None
+        self.f_bias = nn.Parameter(torch.zeros(heads * dim, **f32), requires_grad=False)
+        self.lower = nn.Parameter(torch.zeros(heads * dim, **f32), requires_grad=False)
+        self.norm = nn.Parameter(torch.ones(vdim, **f32), requires_grad=False)
+        self.o = nn.Parameter(torch.empty(width, heads * vdim, dtype=dtype), requires_grad=False)
+
+    @staticmethod
+    def state_shapes(heads: int, dim: int, vdim: int):
+        return {"S": (heads, dim, vdim)}
+
+    def scan(self, a: torch.Tensor, forward_batch: ForwardBatch, state_id: Optional[int] = None) -> torch.Tensor:
+        """a [T, >= in_rows]: the outputs of the rows [q | f | v] -> the mixer's output [T, W]"""
+        seq, states = forward_batch.attn_backend.seq, forward_batch.state_pool
+        nk = self.heads * self.dim
+        S = states.state(self.layer_id if state_id is None else state_id, "S")
+        o = _native.hgrn2_scan(a[:, :nk], a[:, nk:2 * nk], a[:, 2 * nk:self.in_rows], self.f_bias.data, self.lower.data,
+                               self.norm.data, S, seq, self.heads, self.dim, self.vdim, self.eps)
+        return _native.linear(o, self.o)
+
+    def forward(self, h: torch.Tensor, forward_batch: ForwardBatch, state_id: Optional[int] = None) -> torch.Tensor:
+        return self.scan(_native.linear(h, self.in_proj), forward_batch, state_id)

@@ -35,6 +35,11 @@ def _sominex_config(raw: dict, context_len=None, tensor_shapes=None, **_kw):
     return SominexConfig(raw, context_len=context_len or 8192, tensor_shapes=tensor_shapes)
 
 
+def _toredra_config(raw: dict, context_len=None, tensor_shapes=None, **_kw):
+    from .toredra import ToredraConfig
+    return ToredraConfig(raw, context_len=context_len or 8192, tensor_shapes=tensor_shapes)
+
+
 def _llama_class():
     from .llama import LlamaForCausalLM
     return LlamaForCausalLM
@@ -55,12 +60,18 @@ def _sominex_class():
     return SominexForCausalLM
 
 
+def _toredra_class():
+    from .toredra import ToredraForCausalLM
+    return ToredraForCausalLM
+
+
 # architecture name -> (configuration from config.json's dict, model class); both lazy so that naming a model does not
 # import the others
 MODELS = {
     "LlamaForCausalLM": (_llama_config, _llama_class),
     "Tizalorn": (_tizalorn_config, _tizalorn_class),
     "Sominex": (_sominex_config, _sominex_class),
+    "Toredra": (_toredra_config, _toredra_class),
 }
 
 
