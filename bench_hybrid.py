@@ -1,5 +1,6 @@
-"""bench.py --mode hybrid / --mode sominex: prefill and decode throughput of the Tizalorn / the Sominex design at layer sizes
-of real models (random weights), beside a Llama of the same width and depth on the same engine path, and a per-kernel table: every HIP kernel
+"""bench.py --mode hybrid / --mode sominex / --mode toredra: prefill and decode throughput of the Tizalorn / the Sominex / the
+Toredra design at layer sizes of real models (random weights), beside a Llama of the same width and depth on the same engine
+path (the Toredra mode also runs Sominex, its nearest relative), and a per-kernel table: every HIP kernel
 (and library product) of both models timed inside an eager prefill batch and an eager decode step, with the time its
 algorithmic bytes and flops would take at the chip's peaks (fraction of roofline).
 
@@ -52,6 +53,24 @@ def sominex_config(width: int, layers: int, context_len: int):
     raw = {"architecture": "Sominex", "vocab": 128256, "width": width, "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
            "layers": [{**pattern[i % 4][0], "mlp": pattern[i % 4][1]} for i in range(layers)]}
     return SominexConfig(raw, context_len=context_len)
+
+
+def toredra_config(width: int, layers: int, context_len: int):
+    """layers in the order delta, delta, parallel, delta, each with a squared-ReLU feed-forward: delta heads of 64 (rank-64
+    decay projection), attention heads of 128 with a quarter as many key/value heads and rotation on half of each head, beside
+    it a forget-write linear attention of width / 256 heads with 128 x 128 states"""
+    from scratchpad_amd.toredra import ToredraConfig
+    delta = {"type": "general_delta", "mixer": {"heads": width // 64, "dim": 64}}
+    par = {"type": "parallel",
+           "mixer": {"left": {"heads": width // 128, "kv_heads": max(1, width // 512), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                              "rot": {"base": 500000.0, "dims": 64,
+                                      "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 4096}}},
+                     "right": {"heads": max(1, width // 256), "dim": 128, "vdim": 128}}}
+    dense = {"kind": "dense", "ff": {2048: 8192, 4096: 14336}.get(width, 3 * width)}
+    pattern = [delta, delta, par, delta]
+    raw = {"architecture": "Toredra", "vocab": 128256, "width": width, "norm": {"eps": 1e-5}, "logit_scale": 0.5,
+           "logit_softcap": 30.0, "layers": [{**pattern[i % 4], "mlp": dense} for i in range(layers)]}
+    return ToredraConfig(raw, context_len=context_len, decay_rank=64)
 
 
 def llama_config(width: int, layers: int, context_len: int):
@@ -150,6 +169,7 @@ def instrument(clock: KernelClock, cfg):
     def window(a, k, out):
         q, kpool, vpool = a[0], a[1], a[2]
         H, G, D, Dv, size, P = a[7], a[8], a[9], a[10], a[11], a[12]
+        size = size if size > 0 else 1 << 40          # no window: every earlier token
         seen = 0                 # (query, visible key or block) pairs
         for p, e in zip(clock.step["prefix"], clock.step["extend"]):
             for pos in (range(p, p + e) if e <= 4 else ()):
@@ -168,6 +188,14 @@ def instrument(clock: KernelClock, cfg):
         q, S, heads, D, Dv = a[0], a[7], a[11], a[12], a[13]
         return _nbytes(*a[:4], out) + 2 * len(clock.step["extend"]) * heads * D * Dv * 4, 4 * q.shape[0] * heads * D * Dv, VECTOR32
 
+    def delta(a, k, out):        # two sweeps over the state per token: u^T S (2 flops), the update (5), the numerator (2)
+        r, state, heads, dim = a[0], a[7], a[9], a[10]
+        return _nbytes(*a[:6], out) + 2 * len(clock.step["extend"]) * heads * dim * dim * 4, 9 * r.shape[0] * heads * dim * dim, VECTOR32
+
+    def hgrn(a, k, out):         # the update (3 flops per state element and token) and the numerator (2)
+        qpre, state, heads, D, Dv = a[0], a[6], a[8], a[9], a[10]
+        return _nbytes(*a[:3], out) + 2 * len(clock.step["extend"]) * heads * D * Dv * 4, 5 * qpre.shape[0] * heads * D * Dv, VECTOR32
+
     def small(a, k, out):
         x, w = a[0], a[1]
         return _nbytes(x, w, out), 2 * x.shape[0] * w.shape[0] * w.shape[1], VECTOR32
@@ -184,7 +212,9 @@ def instrument(clock: KernelClock, cfg):
              "extend_attention": llama_extend, "decode_attention": llama_extend, "linear": gemm, "linear_silu_mul": gemm,
              "embed_scale": io, "norm_shift": io, "stream_add": io, "qkv_rotary_store": io, "pool_blocks": io,
              "window_attention": window, "small_linear_f32": small, "causal_conv_silu": io, "mamba2_scan": scan,
-             "gated_group_norm": io, "mlstm_scan": mlstm, "moe_route_softmax": io}
+             "gated_group_norm": io, "mlstm_scan": mlstm, "moe_route_softmax": io,
+             "gated_add_norm": io, "relu_square": io, "scale_softcap": io, "delta_gates": io, "delta_recurrence": delta,
+             "hgrn2_scan": hgrn}
     for name, cost in costs.items():
         saved[name] = getattr(N, name)
         setattr(N, name, clock.record(name, saved[name], cost))
@@ -313,7 +343,7 @@ def hybrid_main(args, design: str = "tizalorn"):
     runs = []
     for w in widths:
         row = {"width": w, "layers": layers}
-        for model in (design, "llama"):
+        for model in ((design, "sominex", "llama") if design == "toredra" else (design, "llama")):
             cmd = [sys.executable, "-u", os.path.abspath(__file__), "--child", model, "--width", str(w), "--layers", str(layers),
                    "--bs", str(args.bs), "--ctx", str(args.ctx), "--steps", str(args.steps), "--warmup", str(args.warmup),
                    "--max-prefill-tokens", str(args.max_prefill_tokens)]
@@ -345,7 +375,7 @@ def child_main():
     import sys
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
     ap = argparse.ArgumentParser()
-    ap.add_argument("--child", required=True, choices=["tizalorn", "sominex", "llama"])
+    ap.add_argument("--child", required=True, choices=["tizalorn", "sominex", "toredra", "llama"])
     for name in ("width", "layers", "bs", "ctx", "steps", "warmup", "max-prefill-tokens"):
         ap.add_argument("--" + name, type=int, required=True)
     ap.add_argument("--no-graph", action="store_true")
@@ -355,7 +385,7 @@ def child_main():
         raise SystemExit(DISABLED)
     torch.cuda.set_device(0)
     ctx_len = a.ctx + 2 * (a.steps + a.warmup) + 16
-    cfg = {"sominex": sominex_config, "llama": llama_config}[a.child](a.width, a.layers, ctx_len)
+    cfg = {"sominex": sominex_config, "toredra": toredra_config, "llama": llama_config}[a.child](a.width, a.layers, ctx_len)
     out = run_model(cfg, a, not a.no_kernel_table)
     print("RESULT " + json.dumps(out), flush=True)
 

@@ -18,23 +18,52 @@
 namespace sp {
 namespace {
 
-// w2t: [rank, channels] fp32 (the up-projection transposed: neighbouring threads read neighbouring channels)
-template <typename Tag>
+// w2t: [rank, channels] fp32 (the up-projection transposed: neighbouring threads read neighbouring channels).  A workgroup
+// takes TPB tokens x 256 channels, a thread one channel: every weight it loads serves all TPB tokens (TPB = 8 for prompts'
+// portions), and a step of few tokens (TPB = 1) still spreads over channels / 256 workgroups per token.
+template <typename Tag, int TPB>
 __global__ void __launch_bounds__(kBlock)
 delta_gates_kernel(float* decay, float* remove, const void* p, int64_t p_stride, const float* w2t, const float* w0,
-                   const void* apre, int64_t a_stride, const float* a_bias, int channels, int rank, float rate) {
+                   const void* apre, int64_t a_stride, const float* a_bias, int64_t T, int channels, int rank, float rate) {
   typedef Elem<Tag> E;
-  extern __shared__ float tp[];
-  const int64_t t = blockIdx.x;
-  for (int r = threadIdx.x; r < rank; r += blockDim.x) tp[r] = tanhf(E::load(p, t * p_stride + r));
+  extern __shared__ float tp[];                          // [TPB][rank]
+  const int64_t t0 = (int64_t)blockIdx.x * TPB;
+  const int c = blockIdx.y * kBlock + threadIdx.x;
+  for (int e = threadIdx.x; e < TPB * rank; e += kBlock) {
+    const int tt = e / rank, r = e % rank;
+    tp[e] = t0 + tt < T ? tanhf(E::load(p, (t0 + tt) * p_stride + r)) : 0.f;
+  }
   __syncthreads();
-  for (int c = threadIdx.x; c < channels; c += blockDim.x) {
-    float acc = 0.f;
-    for (int r = 0; r < rank; ++r) acc += w2t[(int64_t)r * channels + c] * tp[r];
-    acc += w0[c];
-    decay[t * channels + c] = expf(-rate / (1.f + expf(-acc)));
-    const float z = E::load(apre, t * a_stride + c) + a_bias[c];
-    remove[t * channels + c] = 1.f / (1.f + expf(-z));
+  if (c >= channels) return;
+  float acc[TPB];
+#pragma unroll
+  for (int tt = 0; tt < TPB; ++tt) acc[tt] = 0.f;
+  int r = 0;
+  for (; r + 4 <= rank; r += 4) {                        // four weights in flight
+    const float w_0 = w2t[(int64_t)r * channels + c], w_1 = w2t[(int64_t)(r + 1) * channels + c];
+    const float w_2 = w2t[(int64_t)(r + 2) * channels + c], w_3 = w2t[(int64_t)(r + 3) * channels + c];
+#pragma unroll
+    for (int tt = 0; tt < TPB; ++tt) {
+      const float* q = tp + tt * rank + r;
+      acc[tt] += w_0 * q[0];
+      acc[tt] += w_1 * q[1];
+      acc[tt] += w_2 * q[2];
+      acc[tt] += w_3 * q[3];
+    }
+  }
+  for (; r < rank; ++r) {
+    const float w = w2t[(int64_t)r * channels + c];
+#pragma unroll
+    for (int tt = 0; tt < TPB; ++tt) acc[tt] += w * tp[tt * rank + r];
+  }
+  const float bias = w0[c], ab = a_bias[c];
+#pragma unroll
+  for (int tt = 0; tt < TPB; ++tt) {
+    const int64_t t = t0 + tt;
+    if (t < T) {
+      decay[t * channels + c] = expf(-rate / (1.f + expf(-(acc[tt] + bias))));
+      remove[t * channels + c] = 1.f / (1.f + expf(-(E::load(apre, t * a_stride + c) + ab)));
+    }
   }
 }
 
@@ -51,7 +80,8 @@ delta_recurrence_kernel(void* out, int64_t out_stride, const void* r, int64_t r_
                         int K, float eps) {
   typedef Elem<Tag> E;
   constexpr int kChunk = delta_chunk(KP), SP = delta_split(KP), DS = KP / SP, ROW = KP + 4 * SP;
-  __shared__ float sr[kChunk][ROW], sk[kChunk][ROW], sw[kChunk][ROW], su[kChunk][ROW], sau[kChunk][ROW];
+  // (rows and parts start at multiples of 16 bytes: the token loop reads them four floats at a time)
+  __shared__ __attribute__((aligned(16))) float sr[kChunk][ROW], sk[kChunk][ROW], sw[kChunk][ROW], su[kChunk][ROW], sau[kChunk][ROW];
   __shared__ float sv[kChunk][KP], so[kChunk][KP], sinv[kChunk];
   const int b = blockIdx.x, h = blockIdx.y, j = threadIdx.x;
   const int nthreads = blockDim.x, wave = j >> 6, lane = j & 63, waves = nthreads >> 6;
@@ -103,23 +133,39 @@ delta_recurrence_kernel(void* out, int64_t out_stride, const void* r, int64_t r_
     }
     __syncthreads();
     for (int tt = 0; tt < n; ++tt) {
-      const float* pu = &su[tt][mine];
-      const float* pau = &sau[tt][mine];
-      const float* pw = &sw[tt][mine];
-      const float* pk = &sk[tt][mine];
-      const float* pr = &sr[tt][mine];
-      float proj = 0.f;
+      const float4* pu = reinterpret_cast<const float4*>(&su[tt][mine]);
+      const float4* pau = reinterpret_cast<const float4*>(&sau[tt][mine]);
+      const float4* pw = reinterpret_cast<const float4*>(&sw[tt][mine]);
+      const float4* pk = reinterpret_cast<const float4*>(&sk[tt][mine]);
+      const float4* pr = reinterpret_cast<const float4*>(&sr[tt][mine]);
+      // (four partial sums per sweep: the chain of dependent additions is a quarter as long; DS is a multiple of 4)
+      float pj[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ii = 0; ii < DS; ++ii) proj += pu[ii] * S[ii];
+      for (int ii = 0; ii < DS; ii += 4) {
+        const float4 u4 = pu[ii / 4];
+        pj[0] += u4.x * S[ii];
+        pj[1] += u4.y * S[ii + 1];
+        pj[2] += u4.z * S[ii + 2];
+        pj[3] += u4.w * S[ii + 3];
+      }
+      float proj = (pj[0] + pj[1]) + (pj[2] + pj[3]);
 #pragma unroll
       for (int off = 1; off < SP; off <<= 1) proj += __shfl_xor(proj, off, 64);
       const float vj = live ? sv[tt][col] : 0.f;
-      float num = 0.f;
+      float nm[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ii = 0; ii < DS; ++ii) {
-        S[ii] = pw[ii] * S[ii] - pau[ii] * proj + pk[ii] * vj;
-        num += S[ii] * pr[ii];
+      for (int ii = 0; ii < DS; ii += 4) {
+        const float4 w4 = pw[ii / 4], a4 = pau[ii / 4], k4 = pk[ii / 4], r4 = pr[ii / 4];
+        S[ii] = w4.x * S[ii] - a4.x * proj + k4.x * vj;
+        S[ii + 1] = w4.y * S[ii + 1] - a4.y * proj + k4.y * vj;
+        S[ii + 2] = w4.z * S[ii + 2] - a4.z * proj + k4.z * vj;
+        S[ii + 3] = w4.w * S[ii + 3] - a4.w * proj + k4.w * vj;
+        nm[0] += S[ii] * r4.x;
+        nm[1] += S[ii + 1] * r4.y;
+        nm[2] += S[ii + 2] * r4.z;
+        nm[3] += S[ii + 3] * r4.w;
       }
+      float num = (nm[0] + nm[1]) + (nm[2] + nm[3]);
 #pragma unroll
       for (int off = 1; off < SP; off <<= 1) num += __shfl_xor(num, off, 64);
       if (live && part == 0) so[tt][col] = num;
@@ -183,9 +229,16 @@ extern "C" int sp_delta_gates(float* decay, float* remove, const void* p, int64_
   SP_CHECK_ARG(num_tokens >= 0 && channels > 0 && rank > 0 && rank <= 8192);
   if (num_tokens == 0) return SP_OK;
   SP_CHECK_ARG(decay && remove && p && w2t && w0 && apre && a_bias && p_stride >= rank && a_stride >= channels);
-  SP_DISPATCH_DTYPE(dtype, (delta_gates_kernel<Tag><<<dim3((unsigned)num_tokens), kBlock, rank * sizeof(float),
-                                                       (hipStream_t)stream>>>(decay, remove, p, p_stride, w2t, w0, apre,
-                                                                              a_stride, a_bias, channels, rank, rate)));
+  const unsigned cb = (unsigned)((channels + kBlock - 1) / kBlock);
+  if (num_tokens >= 64 && rank <= 1024) {
+    SP_DISPATCH_DTYPE(dtype, (delta_gates_kernel<Tag, 8><<<dim3((unsigned)((num_tokens + 7) / 8), cb), kBlock,
+                                                            8 * rank * sizeof(float), (hipStream_t)stream>>>(
+                                 decay, remove, p, p_stride, w2t, w0, apre, a_stride, a_bias, num_tokens, channels, rank, rate)));
+  } else {
+    SP_DISPATCH_DTYPE(dtype, (delta_gates_kernel<Tag, 1><<<dim3((unsigned)num_tokens, cb), kBlock, rank * sizeof(float),
+                                                            (hipStream_t)stream>>>(
+                                 decay, remove, p, p_stride, w2t, w0, apre, a_stride, a_bias, num_tokens, channels, rank, rate)));
+  }
   SP_LAUNCH_CHECK();
   return SP_OK;
 }

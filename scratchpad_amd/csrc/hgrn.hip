@@ -23,7 +23,9 @@ hgrn2_scan_kernel(void* out, int64_t out_stride, const void* qpre, int64_t q_str
                   int64_t state_stride, SeqBatch s, int H, int D, int Dv, float eps) {
   typedef Elem<Tag> E;
   constexpr int kChunk = hgrn_chunk(DP), SP = hgrn_split(DP), DS = DP / SP, ROW = DP + 4 * SP;
-  __shared__ float sq[kChunk][ROW], sf[kChunk][ROW], sinv[kChunk];
+  // (rows and parts start at multiples of 16 bytes: the token loop reads them four floats at a time)
+  __shared__ __attribute__((aligned(16))) float sq[kChunk][ROW], sf[kChunk][ROW];
+  __shared__ float sinv[kChunk];
   extern __shared__ float so[];                         // [kChunk][Dv] numerators, then [kChunk][Dv] values
   float* sv = so + (size_t)kChunk * Dv;
   const int b = blockIdx.x, h = blockIdx.y, j = threadIdx.x;
@@ -66,16 +68,23 @@ hgrn2_scan_kernel(void* out, int64_t out_stride, const void* qpre, int64_t q_str
     }
     __syncthreads();
     for (int tt = 0; tt < n; ++tt) {
-      const float* pf = &sf[tt][mine];
-      const float* pq = &sq[tt][mine];
+      const float4* pf = reinterpret_cast<const float4*>(&sf[tt][mine]);
+      const float4* pq = reinterpret_cast<const float4*>(&sq[tt][mine]);
       const float vj = live ? sv[tt * Dv + col] : 0.f;
-      float num = 0.f;
+      float nm[4] = {0.f, 0.f, 0.f, 0.f};          // four partial sums: a quarter of the chain of dependent additions
 #pragma unroll
-      for (int ii = 0; ii < DS; ++ii) {
-        const float f = pf[ii];
-        S[ii] = f * S[ii] + (1.f - f) * vj;
-        num += S[ii] * pq[ii];
+      for (int ii = 0; ii < DS; ii += 4) {
+        const float4 f4 = pf[ii / 4], q4 = pq[ii / 4];
+        S[ii] = f4.x * S[ii] + (1.f - f4.x) * vj;
+        S[ii + 1] = f4.y * S[ii + 1] + (1.f - f4.y) * vj;
+        S[ii + 2] = f4.z * S[ii + 2] + (1.f - f4.z) * vj;
+        S[ii + 3] = f4.w * S[ii + 3] + (1.f - f4.w) * vj;
+        nm[0] += S[ii] * q4.x;
+        nm[1] += S[ii + 1] * q4.y;
+        nm[2] += S[ii + 2] * q4.z;
+        nm[3] += S[ii + 3] * q4.w;
       }
+      float num = (nm[0] + nm[1]) + (nm[2] + nm[3]);
 #pragma unroll
       for (int off = 1; off < SP; off <<= 1) num += __shfl_xor(num, off, 64);
       if (live && part == 0) so[tt * Dv + col] = num;
