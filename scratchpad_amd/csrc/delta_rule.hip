@@ -68,10 +68,13 @@ delta_gates_kernel(float* decay, float* remove, const void* p, int64_t p_stride,
 }
 
 constexpr int delta_chunk(int KP) { return KP > 64 ? 8 : 16; }                      // tokens staged in LDS per pass
-constexpr int delta_split(int KP) { return KP > 64 ? 4 : (KP > 32 ? 2 : 1); }       // lanes that share one column of S
+constexpr int delta_split(int KP) { return KP > 32 ? 4 : (KP > 16 ? 2 : 1); }       // lanes that share one column of S
 
 // thread = (column col of S, part): part p of SP owns the rows [p DS, (p + 1) DS) of the column.  LDS rows are padded by
 // 4 floats per part so that the parts' simultaneous broadcast reads fall into different banks.
+// A pass's operands come from global memory into registers in ONE burst (every load issued before the first is used), and
+// the burst of pass n + 1 is issued right before the token loop of pass n, so it flies while the recurrence runs; the loop
+// itself touches LDS and registers only.
 template <typename Tag, int KP>
 __global__ void __launch_bounds__(KP * delta_split(KP) < 64 ? 64 : KP * delta_split(KP))
 delta_recurrence_kernel(void* out, int64_t out_stride, const void* r, int64_t r_stride, const void* k, int64_t k_stride,
@@ -80,11 +83,14 @@ delta_recurrence_kernel(void* out, int64_t out_stride, const void* r, int64_t r_
                         int K, float eps) {
   typedef Elem<Tag> E;
   constexpr int kChunk = delta_chunk(KP), SP = delta_split(KP), DS = KP / SP, ROW = KP + 4 * SP;
+  constexpr int NT = KP * SP < 64 ? 64 : KP * SP;       // threads of the workgroup (the launch uses exactly these)
+  constexpr int TSTEP = NT / KP, PER = kChunk / TSTEP;  // staging: thread j takes channel j % KP of tokens j / KP + u TSTEP
+  constexpr int PERG = kChunk / SP;                     // epilogue: thread (col, part) takes tokens part + u SP
   // (rows and parts start at multiples of 16 bytes: the token loop reads them four floats at a time)
   __shared__ __attribute__((aligned(16))) float sr[kChunk][ROW], sk[kChunk][ROW], sw[kChunk][ROW], su[kChunk][ROW], sau[kChunk][ROW];
   __shared__ float sv[kChunk][KP], so[kChunk][KP], sinv[kChunk];
   const int b = blockIdx.x, h = blockIdx.y, j = threadIdx.x;
-  const int nthreads = blockDim.x, wave = j >> 6, lane = j & 63, waves = nthreads >> 6;
+  const int wave = j >> 6, lane = j & 63, waves = NT >> 6;
   const int col = j / SP, part = j % SP;
   int64_t start, len, prefix;
   seq_span(s, b, start, len, prefix);
@@ -92,27 +98,53 @@ delta_recurrence_kernel(void* out, int64_t out_stride, const void* r, int64_t r_
   const bool live = col < K;
   float* st = state + load_idx(s.req_pool_indices, b, s.idx64) * state_stride + (int64_t)h * K * K;
   const bool held = prefix > 0;
+  const int64_t hc = (int64_t)h * K, HK = (int64_t)H * K;
+  const int mine = part * (DS + 4);
+  const int si = j % KP, st0 = j / KP;                  // this thread's staged channel and first staged token
+  const bool sok = si < K;
+  const int sat = si + 4 * (si / DS);
+  float fr[PER], fk[PER], fw[PER], fa[PER], fv[PER], fg[PERG];
+  // the operands of the pass that starts at c0 (rows past the pass's end repeat its last row; they are never used)
+  auto fetch = [&](int64_t c0) {
+    const int n = (int)(len - c0 < kChunk ? len - c0 : kChunk);
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      const int tt = st0 + u * TSTEP;
+      const int64_t row = start + c0 + (tt < n ? tt : n - 1);
+      fr[u] = sok ? E::load(r, row * r_stride + hc + si) : 0.f;
+      fk[u] = sok ? E::load(k, row * k_stride + hc + si) : 0.f;
+      fv[u] = sok ? E::load(v, row * v_stride + hc + si) : 0.f;
+      fw[u] = sok ? decay[row * HK + hc + si] : 0.f;
+      fa[u] = sok ? remove[row * HK + hc + si] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < PERG; ++u) {
+      const int tt = part + u * SP;
+      fg[u] = live ? E::load(g, (start + c0 + (tt < n ? tt : n - 1)) * g_stride + hc + col) : 0.f;
+    }
+  };
+  fetch(0);
   float S[DS];
 #pragma unroll
   for (int ii = 0; ii < DS; ++ii) {
     const int i = part * DS + ii;
     S[ii] = (live && i < K && held) ? st[(int64_t)i * K + col] : 0.f;
   }
-  const int64_t hc = (int64_t)h * K, HK = (int64_t)H * K;
-  const int mine = part * (DS + 4);
+  const float nw = live ? norm_w[hc + col] : 0.f;
   for (int64_t c0 = 0; c0 < len; c0 += kChunk) {
     const int n = (int)(len - c0 < kChunk ? len - c0 : kChunk);
-    __syncthreads();
-    for (int e = j; e < n * KP; e += nthreads) {
-      const int tt = e / KP, i = e % KP;
-      const int64_t row = start + c0 + tt;
-      const bool ok = i < K;
-      const int at = i + 4 * (i / DS);
-      sr[tt][at] = ok ? E::load(r, row * r_stride + hc + i) : 0.f;
-      sk[tt][at] = ok ? E::load(k, row * k_stride + hc + i) : 0.f;
-      sw[tt][at] = ok ? decay[row * HK + hc + i] : 0.f;
-      sau[tt][at] = ok ? remove[row * HK + hc + i] : 0.f;
-      sv[tt][i] = ok ? E::load(v, row * v_stride + hc + i) : 0.f;
+    __syncthreads();                                     // the previous pass's epilogue is done with so and sinv
+    float gate[PERG];
+#pragma unroll
+    for (int u = 0; u < PERG; ++u) gate[u] = fg[u];
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      const int tt = st0 + u * TSTEP;
+      sr[tt][sat] = fr[u];
+      sk[tt][sat] = fk[u];
+      sw[tt][sat] = fw[u];
+      sau[tt][sat] = fa[u];
+      sv[tt][si] = fv[u];
     }
     __syncthreads();
     // the unit key of every token of the pass: a wave per token
@@ -132,6 +164,7 @@ delta_recurrence_kernel(void* out, int64_t out_stride, const void* r, int64_t r_
       }
     }
     __syncthreads();
+    if (c0 + kChunk < len) fetch(c0 + kChunk);           // in flight while the recurrence runs
     for (int tt = 0; tt < n; ++tt) {
       const float4* pu = reinterpret_cast<const float4*>(&su[tt][mine]);
       const float4* pau = reinterpret_cast<const float4*>(&sau[tt][mine]);
@@ -180,11 +213,11 @@ delta_recurrence_kernel(void* out, int64_t out_stride, const void* r, int64_t r_
     }
     __syncthreads();
     if (live) {
-      const float nw = norm_w[hc + col];
-      for (int tt = part; tt < n; tt += SP) {
-        const int64_t row = start + c0 + tt;
-        const float gv = E::load(g, row * g_stride + hc + col);
-        E::store(out, row * out_stride + hc + col, so[tt][col] * sinv[tt] * nw / (1.f + expf(-gv)));
+#pragma unroll
+      for (int u = 0; u < PERG; ++u) {
+        const int tt = part + u * SP;
+        if (tt < n)
+          E::store(out, (start + c0 + tt) * out_stride + hc + col, so[tt][col] * sinv[tt] * nw / (1.f + expf(-gate[u])));
       }
     }
   }
@@ -204,7 +237,7 @@ static int launch_delta(void* out, int64_t out_stride, const void* r, int64_t r_
                         int H, int K, float eps, hipStream_t st) {
   const dim3 grid((unsigned)s.B, (unsigned)H);
 #define SP_DELTA(KP)                                                                                                    \
-  delta_recurrence_kernel<Tag, KP><<<grid, (unsigned)((K * delta_split(KP) + 63) / 64 * 64), 0, st>>>(                  \
+  delta_recurrence_kernel<Tag, KP><<<grid, (unsigned)(KP * delta_split(KP) < 64 ? 64 : KP * delta_split(KP)), 0, st>>>(  \
       out, out_stride, r, r_stride, k, k_stride, v, v_stride, g, g_stride, decay, remove, norm_w, state, state_stride, s, H, K, \
       eps)
   if (K <= 16) SP_DELTA(16);

@@ -16,20 +16,25 @@ namespace {
 constexpr int hgrn_chunk(int DP) { return DP > 128 ? 8 : 16; }
 constexpr int hgrn_split(int DP) { return DP > 64 ? 4 : (DP > 32 ? 2 : 1); }
 
-template <typename Tag, int DP>
-__global__ void __launch_bounds__(256 * hgrn_split(DP))
+// A pass's operands come from global memory into registers in ONE burst (every load issued before the first is used), and
+// the burst of pass n + 1 is issued right before the token loop of pass n, so it flies while the recurrence runs; the loop
+// itself touches LDS and registers only.  NT threads: Dv columns x SP parts, rounded up to whole waves.
+template <typename Tag, int DP, int NT>
+__global__ void __launch_bounds__(NT)
 hgrn2_scan_kernel(void* out, int64_t out_stride, const void* qpre, int64_t q_stride, const void* fpre, int64_t f_stride,
                   const void* v, int64_t v_stride, const float* f_bias, const float* lower, const float* norm_w, float* state,
                   int64_t state_stride, SeqBatch s, int H, int D, int Dv, float eps) {
   typedef Elem<Tag> E;
   constexpr int kChunk = hgrn_chunk(DP), SP = hgrn_split(DP), DS = DP / SP, ROW = DP + 4 * SP;
+  constexpr int PERK = (kChunk * DP + NT - 1) / NT;     // staged (token, query channel) elements per thread and pass
+  constexpr int PERV = kChunk / SP;                     // value / output tokens per thread: tokens part + u SP of column col
   // (rows and parts start at multiples of 16 bytes: the token loop reads them four floats at a time)
   __shared__ __attribute__((aligned(16))) float sq[kChunk][ROW], sf[kChunk][ROW];
   __shared__ float sinv[kChunk];
   extern __shared__ float so[];                         // [kChunk][Dv] numerators, then [kChunk][Dv] values
   float* sv = so + (size_t)kChunk * Dv;
   const int b = blockIdx.x, h = blockIdx.y, j = threadIdx.x;
-  const int nthreads = blockDim.x, wave = j >> 6, lane = j & 63, waves = nthreads >> 6;
+  const int wave = j >> 6, lane = j & 63, waves = NT >> 6;
   const int col = j / SP, part = j % SP;
   int64_t start, len, prefix;
   seq_span(s, b, start, len, prefix);
@@ -37,36 +42,62 @@ hgrn2_scan_kernel(void* out, int64_t out_stride, const void* qpre, int64_t q_str
   const bool live = col < Dv;
   float* st = state + load_idx(s.req_pool_indices, b, s.idx64) * state_stride + (int64_t)h * D * Dv;
   const bool held = prefix > 0;
+  const int64_t colk = (int64_t)h * D, colv = (int64_t)h * Dv;
+  const int mine = part * (DS + 4);
+  float fq[PERK], ff[PERK], fvv[PERV];
+  // the operands of the pass that starts at c0 (rows past the pass's end repeat its last row; they are never used)
+  auto fetch = [&](int64_t c0) {
+    const int n = (int)(len - c0 < kChunk ? len - c0 : kChunk);
+#pragma unroll
+    for (int u = 0; u < PERK; ++u) {
+      const int e = j + u * NT, tt = e / DP, i = e % DP;
+      const bool ok = e < kChunk * DP && i < D;
+      const int64_t row = start + c0 + (tt < n ? tt : n - 1);
+      fq[u] = ok ? E::load(qpre, row * q_stride + colk + i) : 0.f;
+      ff[u] = ok ? E::load(fpre, row * f_stride + colk + i) : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < PERV; ++u) {
+      const int tt = part + u * SP;
+      fvv[u] = live ? E::load(v, (start + c0 + (tt < n ? tt : n - 1)) * v_stride + colv + col) : 0.f;
+    }
+  };
+  fetch(0);
   float S[DS];
 #pragma unroll
   for (int ii = 0; ii < DS; ++ii) {
     const int i = part * DS + ii;
     S[ii] = (live && i < D && held) ? st[(int64_t)i * Dv + col] : 0.f;
   }
-  const int64_t colk = (int64_t)h * D, colv = (int64_t)h * Dv;
-  const int mine = part * (DS + 4);
+  // gate constants of this thread's staged channels (the same channel in every pass)
+  float flo[PERK], fbi[PERK];
+#pragma unroll
+  for (int u = 0; u < PERK; ++u) {
+    const int e = j + u * NT, i = e % DP;
+    const bool ok = e < kChunk * DP && i < D;
+    flo[u] = ok ? lower[colk + i] : 0.f;
+    fbi[u] = ok ? f_bias[colk + i] : 0.f;
+  }
+  const float nw = live ? norm_w[col] : 0.f;
   for (int64_t c0 = 0; c0 < len; c0 += kChunk) {
     const int n = (int)(len - c0 < kChunk ? len - c0 : kChunk);
-    __syncthreads();
-    for (int e = j; e < n * DP; e += nthreads) {
-      const int tt = e / DP, i = e % DP;
-      const int64_t row = start + c0 + tt;
-      const int at = i + 4 * (i / DS);
-      float qv = 0.f, fv = 0.f;
-      if (i < D) {
-        const float z = E::load(qpre, row * q_stride + colk + i);
-        qv = z / (1.f + expf(-z));
-        const float lo = lower[colk + i];
-        fv = lo + (1.f - lo) / (1.f + expf(-(E::load(fpre, row * f_stride + colk + i) + f_bias[colk + i])));
+    __syncthreads();                                     // the previous pass's epilogue is done with so and sinv
+#pragma unroll
+    for (int u = 0; u < PERK; ++u) {
+      const int e = j + u * NT, tt = e / DP, i = e % DP;
+      if (e < kChunk * DP) {
+        const int at = i + 4 * (i / DS);
+        const bool ok = i < D;                           // register rows past D: f = 0 and q = 0, never stored
+        sq[tt][at] = ok ? fq[u] / (1.f + expf(-fq[u])) : 0.f;
+        sf[tt][at] = ok ? flo[u] + (1.f - flo[u]) / (1.f + expf(-(ff[u] + fbi[u]))) : 0.f;
       }
-      sq[tt][at] = qv;
-      sf[tt][at] = fv;
     }
-    for (int e = j; e < n * Dv; e += nthreads) {
-      const int tt = e / Dv, c = e % Dv;
-      sv[tt * Dv + c] = E::load(v, (start + c0 + tt) * v_stride + colv + c);
+    if (live) {
+#pragma unroll
+      for (int u = 0; u < PERV; ++u) sv[(part + u * SP) * Dv + col] = fvv[u];
     }
     __syncthreads();
+    if (c0 + kChunk < len) fetch(c0 + kChunk);           // in flight while the recurrence runs
     for (int tt = 0; tt < n; ++tt) {
       const float4* pf = reinterpret_cast<const float4*>(&sf[tt][mine]);
       const float4* pq = reinterpret_cast<const float4*>(&sq[tt][mine]);
@@ -98,9 +129,11 @@ hgrn2_scan_kernel(void* out, int64_t out_stride, const void* qpre, int64_t q_str
     }
     __syncthreads();
     if (live) {
-      const float nw = norm_w[col];
-      for (int tt = part; tt < n; tt += SP)
-        E::store(out, (start + c0 + tt) * out_stride + colv + col, so[tt * Dv + col] * sinv[tt] * nw);
+#pragma unroll
+      for (int u = 0; u < PERV; ++u) {
+        const int tt = part + u * SP;
+        if (tt < n) E::store(out, (start + c0 + tt) * out_stride + colv + col, so[tt * Dv + col] * sinv[tt] * nw);
+      }
     }
   }
   if (live) {
@@ -120,10 +153,19 @@ static int launch_hgrn2(void* out, int64_t out_stride, const void* qpre, int64_t
   const dim3 grid((unsigned)s.B, (unsigned)H);
   if (Dv * (D > 64 ? 4 : (D > 32 ? 2 : 1)) > 1024) return SP_ERR_UNSUPPORTED;
   // (register rows past D take f = 0 and q = 0: whatever they hold never reaches an output and is never stored)
-#define SP_HGRN(DP)                                                                                                     \
-  hgrn2_scan_kernel<Tag, DP><<<grid, (unsigned)((Dv * hgrn_split(DP) + 63) / 64 * 64),                                  \
-                               (size_t)hgrn_chunk(DP) * 2 * Dv * sizeof(float), st>>>(                                  \
+  // workgroup sizes come in steps (the staging's trip count is a compile-time number): the next one that holds Dv columns
+#define SP_HGRN_NT(DP, NT)                                                                                              \
+  hgrn2_scan_kernel<Tag, DP, NT><<<grid, NT, (size_t)hgrn_chunk(DP) * 2 * Dv * sizeof(float), st>>>(                    \
       out, out_stride, qpre, q_stride, fpre, f_stride, v, v_stride, f_bias, lower, norm_w, state, state_stride, s, H, D, Dv, eps)
+#define SP_HGRN(DP)                                                                                                     \
+  do {                                                                                                                  \
+    const int need = Dv * hgrn_split(DP);                                                                               \
+    if (need <= 64) SP_HGRN_NT(DP, 64);                                                                                 \
+    else if (need <= 128) SP_HGRN_NT(DP, 128);                                                                          \
+    else if (need <= 256) SP_HGRN_NT(DP, 256);                                                                          \
+    else if (need <= 512) SP_HGRN_NT(DP, 512);                                                                          \
+    else SP_HGRN_NT(DP, 1024);                                                                                          \
+  } while (0)
   if (D <= 16) SP_HGRN(16);
   else if (D <= 32) SP_HGRN(32);
   else if (D <= 64) SP_HGRN(64);
@@ -131,6 +173,7 @@ static int launch_hgrn2(void* out, int64_t out_stride, const void* qpre, int64_t
   else if (D <= 256) SP_HGRN(256);
   else return SP_ERR_UNSUPPORTED;
 #undef SP_HGRN
+#undef SP_HGRN_NT
   SP_LAUNCH_CHECK();
   return SP_OK;
 }
