@@ -8,7 +8,7 @@
 //   w = exp(-rate * sigmoid(W2 tanh(p) + w0))            (p = the low-rank projection's output)
 //   a = sigmoid(apre + a_bias)
 //
-// One workgroup per (request, head): a column of S (one value channel) lives in the registers of 1, 2 or 4 neighbouring
+// One workgroup per (request, head): a column of S (one value channel) lives in the registers of 2, 4 or 8 neighbouring
 // lanes; the request's tokens of this step are walked in order from the state the previous step left in the pool (zeros
 // at a sequence's first token), staged through LDS in passes.  A token costs two sweeps over the column - u^T S first,
 // then the update with the numerator - and two lane exchanges, no workgroup barrier.  Prompt portions and single decoded
@@ -68,7 +68,10 @@ delta_gates_kernel(float* decay, float* remove, const void* p, int64_t p_stride,
 }
 
 constexpr int delta_chunk(int KP) { return KP > 64 ? 8 : 16; }                      // tokens staged in LDS per pass
-constexpr int delta_split(int KP) { return KP > 32 ? 4 : (KP > 16 ? 2 : 1); }       // lanes that share one column of S
+// lanes that share one column of S: 8 state values per lane where the workgroup's 1024 threads allow it (measured at heads of
+// 64: 2 lanes 1.07 ms, 4 lanes 0.58 ms, 8 lanes 0.38 ms, 16 lanes 0.49 ms per 4096 tokens - more waves per SIMD hide the
+// waits of the per-token chain until the lane exchanges take over)
+constexpr int delta_split(int KP) { return KP > 128 ? 4 : (KP > 32 ? 8 : (KP > 16 ? 4 : 2)); }
 
 // thread = (column col of S, part): part p of SP owns the rows [p DS, (p + 1) DS) of the column.  LDS rows are padded by
 // 4 floats per part so that the parts' simultaneous broadcast reads fall into different banks.

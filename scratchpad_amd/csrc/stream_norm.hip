@@ -147,6 +147,146 @@ gated_add_norm_kernel(float* x, int64_t x_stride, const void* a, int64_t a_strid
   for (int i = threadIdx.x; i < width; i += blockDim.x) E::store(out_next, t * next_stride + i, rowbuf[i] * invx * next_weight[i]);
 }
 
+// The same on 16-byte vectors, for rows of NV x 256 vectors at most: a thread holds its part of the row in registers, every
+// activation it needs (a, b, gate, x, extra) is loaded before the first reduction, and the three norms follow one another
+// without a further pass over memory.
+template <typename Tag, int NV>
+__global__ void __launch_bounds__(kBlock)
+gated_add_norm_vec_kernel(float* x, int64_t x_stride, const void* a, int64_t a_stride, const float* wa, const void* b,
+                          int64_t b_stride, const float* wb, const void* gate, int64_t gate_stride, const float* gate_bias,
+                          const float* weight, const float* extra, int64_t extra_stride, void* out_next, int64_t next_stride,
+                          const float* next_weight, int width, float eps) {
+  typedef Elem<Tag> E;
+  constexpr int V = E::kVec;
+  __shared__ float red[2 * (kBlock / 64)];
+  const int64_t t = blockIdx.x;
+  const int nvec = width / V;
+  float ya[NV][V], yb[NV][V], yg[NV][V], xs[NV][V];
+#pragma unroll
+  for (int u = 0; u < NV; ++u) {
+    const int vi = threadIdx.x + u * kBlock;
+    const bool on = vi < nvec;
+    const int64_t c = (int64_t)vi * V;
+    if (on) {
+      unpack16<Tag>(ld16((const char*)a + (t * a_stride + c) * E::kBytes), ya[u]);
+      if (b) unpack16<Tag>(ld16((const char*)b + (t * b_stride + c) * E::kBytes), yb[u]);
+      if (gate) unpack16<Tag>(ld16((const char*)gate + (t * gate_stride + c) * E::kBytes), yg[u]);
+#pragma unroll
+      for (int q = 0; q < V / 4; ++q) {
+        unpack16<f32_tag>(ld16(x + t * x_stride + c + 4 * q), xs[u] + 4 * q);
+        if (extra) {
+          float ex[4];
+          unpack16<f32_tag>(ld16(extra + t * extra_stride + c + 4 * q), ex);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) xs[u][4 * q + e] += ex[e];
+        }
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; ++e) ya[u][e] = yb[u][e] = yg[u][e] = xs[u][e] = 0.f;
+    }
+  }
+  auto sum2 = [&](float& p, float& q) {           // two sums over the workgroup at once
+    p = wave_sum(p);
+    q = wave_sum(q);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    __syncthreads();
+    if (lane == 0) {
+      red[2 * wave] = p;
+      red[2 * wave + 1] = q;
+    }
+    __syncthreads();
+    p = q = 0.f;
+    for (int w = 0; w < kBlock / 64; ++w) {
+      p += red[2 * w];
+      q += red[2 * w + 1];
+    }
+  };
+  auto row4 = [&](const float* w, int64_t c, float* f) { unpack16<f32_tag>(ld16(w + c), f); };
+  if (b) {
+    float sa = 0.f, sb = 0.f;
+#pragma unroll
+    for (int u = 0; u < NV; ++u)
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        sa += ya[u][e] * ya[u][e];
+        sb += yb[u][e] * yb[u][e];
+      }
+    sum2(sa, sb);
+    const float ia = 1.f / sqrtf(sa / (float)width + eps), ib = 1.f / sqrtf(sb / (float)width + eps);
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int vi = threadIdx.x + u * kBlock;
+      if (vi < nvec) {
+#pragma unroll
+        for (int q = 0; q < V / 4; ++q) {
+          float fa[4], fb[4];
+          row4(wa, (int64_t)vi * V + 4 * q, fa);
+          row4(wb, (int64_t)vi * V + 4 * q, fb);
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            ya[u][4 * q + e] = 0.5f * (ya[u][4 * q + e] * ia * fa[e] + yb[u][4 * q + e] * ib * fb[e]);
+        }
+      }
+    }
+  }
+  float ss = 0.f, unused = 0.f;
+#pragma unroll
+  for (int u = 0; u < NV; ++u) {
+    const int vi = threadIdx.x + u * kBlock;
+    if (gate && vi < nvec) {
+#pragma unroll
+      for (int q = 0; q < V / 4; ++q) {
+        float gb[4] = {0.f, 0.f, 0.f, 0.f};
+        if (gate_bias) row4(gate_bias, (int64_t)vi * V + 4 * q, gb);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) ya[u][4 * q + e] /= 1.f + expf(-(yg[u][4 * q + e] + gb[e]));
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < V; ++e) ss += ya[u][e] * ya[u][e];
+  }
+  sum2(ss, unused);
+  const float inv = 1.f / sqrtf(ss / (float)width + eps);
+  float sx = 0.f;
+#pragma unroll
+  for (int u = 0; u < NV; ++u) {
+    const int vi = threadIdx.x + u * kBlock;
+    if (vi < nvec) {
+#pragma unroll
+      for (int q = 0; q < V / 4; ++q) {
+        float fw[4];
+        row4(weight, (int64_t)vi * V + 4 * q, fw);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          xs[u][4 * q + e] += ya[u][4 * q + e] * inv * fw[e];      // (the pass's added rows joined x when it was loaded)
+        }
+        st16(x + t * x_stride + (int64_t)vi * V + 4 * q, pack16<f32_tag>(xs[u] + 4 * q));
+      }
+#pragma unroll
+      for (int e = 0; e < V; ++e) sx += xs[u][e] * xs[u][e];
+    }
+  }
+  if (!out_next) return;
+  sum2(sx, unused);
+  const float invx = 1.f / sqrtf(sx / (float)width + eps);
+#pragma unroll
+  for (int u = 0; u < NV; ++u) {
+    const int vi = threadIdx.x + u * kBlock;
+    if (vi < nvec) {
+      float o[V];
+#pragma unroll
+      for (int q = 0; q < V / 4; ++q) {
+        float fw[4];
+        row4(next_weight, (int64_t)vi * V + 4 * q, fw);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[4 * q + e] = xs[u][4 * q + e] * invx * fw[e];
+      }
+      st16((char*)out_next + (t * next_stride + (int64_t)vi * V) * E::kBytes, pack16<Tag>(o));
+    }
+  }
+}
+
 }  // namespace
 }  // namespace sp
 
@@ -217,6 +357,28 @@ extern "C" int sp_gated_add_norm(float* x, int64_t x_stride, const void* a, int6
   SP_CHECK_ARG(!gate || gate_stride >= width);
   SP_CHECK_ARG(!extra || extra_stride >= width);
   SP_CHECK_ARG(!out_next || (next_weight && next_stride >= width));
+  // rows of 16-byte vectors that 256 threads hold in registers: the vector kernel; anything else: the scalar one
+  const int vecn = dtype == SP_F32 ? 4 : 8, esize = dtype == SP_F32 ? 4 : 2;
+  auto al = [&](const void* p, int64_t stride, int elem_bytes) {
+    return !p || ((((uintptr_t)p) & 15) == 0 && (stride * elem_bytes) % 16 == 0);
+  };
+  const bool vec = width % vecn == 0 && width / vecn <= 4 * kBlock && al(x, x_stride, 4) && al(a, a_stride, esize) &&
+                   al(b, b_stride, esize) && al(gate, gate_stride, esize) && al(extra, extra_stride, 4) &&
+                   al(out_next, next_stride, esize) && al(weight, 0, 4) && al(wa, 0, 4) && al(wb, 0, 4) && al(gate_bias, 0, 4) &&
+                   al(next_weight, 0, 4);
+  if (vec) {
+    const int nv = (width / vecn + kBlock - 1) / kBlock;
+#define SP_GAN(NV)                                                                                                      \
+  SP_DISPATCH_DTYPE(dtype, (gated_add_norm_vec_kernel<Tag, NV><<<dim3((unsigned)num_tokens), kBlock, 0, (hipStream_t)stream>>>( \
+                               x, x_stride, a, a_stride, wa, b, b_stride, wb, gate, gate_stride, gate_bias, weight, extra,  \
+                               extra_stride, out_next, next_stride, next_weight, width, eps)))
+    if (nv <= 1) SP_GAN(1);
+    else if (nv <= 2) SP_GAN(2);
+    else SP_GAN(4);
+#undef SP_GAN
+    SP_LAUNCH_CHECK();
+    return SP_OK;
+  }
   SP_DISPATCH_DTYPE(dtype, (gated_add_norm_kernel<Tag><<<dim3((unsigned)num_tokens), kBlock, (size_t)width * sizeof(float),
                                                           (hipStream_t)stream>>>(
                                x, x_stride, a, a_stride, wa, b, b_stride, wb, gate, gate_stride, gate_bias, weight, extra,

@@ -88,10 +88,12 @@ def test_single_layer_models_match_oracle(tmp_path, layer):
 
 
 # ------------------------------------------------------------------------------------------------ row kernels
-def test_gated_add_norm_kernel_in_every_form():
+@pytest.mark.parametrize("W", [200, 77, 3000], ids=["vectors", "scalars", "several-vectors-per-thread"])
+def test_gated_add_norm_kernel_in_every_form(W):
+    """rows of whole 16-byte vectors stay in registers; other widths take the scalar kernel"""
     from scratchpad_amd import _native
     g = torch.Generator().manual_seed(0)
-    T, W, eps = 37, 200, 1e-5
+    T, eps = 37, 1e-5
     rn = lambda *s: torch.randn(*s, generator=g)
     x, a, b, gate, extra = rn(T, W), rn(T, W) * 3, rn(T, W) * 0.2, rn(T, 2 * W), rn(T, W)
     w, wa, wb, gb, nw = (1 + 0.3 * rn(W) for _ in range(5))
