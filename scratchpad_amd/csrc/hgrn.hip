@@ -5,7 +5,7 @@
 //   out = o / rms_head(o) * norm_w         (norm_w [Dv], the same for every head)
 // There is no key: the row of S that belongs to query channel i takes in (1 - f_i) of the value.
 //
-// One workgroup per (request, head): a column of S (one value channel) lives in the registers of 1, 2 or 4 neighbouring
+// One workgroup per (request, head): a column of S (one value channel) lives in the registers of 1 to 8 neighbouring
 // lanes; the request's tokens of this step are walked in order from the state the previous step left in the pool (zeros at
 // a sequence's first token), staged through LDS in passes of 16 tokens, the head norm as the pass's epilogue.
 #include "seq_batch.h"
@@ -14,18 +14,21 @@ namespace sp {
 namespace {
 
 constexpr int hgrn_chunk(int DP) { return DP > 128 ? 8 : 16; }
-constexpr int hgrn_split(int DP) { return DP > 64 ? 4 : (DP > 32 ? 2 : 1); }
+// lanes that share one column of S: 8 state values per lane (more waves per SIMD fill the waits of a wave's per-token chain)
+// where the workgroup's 1024 threads hold vdim columns of that many lanes, else the coarser split that always fits
+constexpr int hgrn_split_fine(int DP) { return DP / 8 > 8 ? 8 : DP / 8; }
+constexpr int hgrn_split_coarse(int DP) { return DP > 64 ? 4 : (DP > 32 ? 2 : 1); }
 
 // A pass's operands come from global memory into registers in ONE burst (every load issued before the first is used), and
 // the burst of pass n + 1 is issued right before the token loop of pass n, so it flies while the recurrence runs; the loop
 // itself touches LDS and registers only.  NT threads: Dv columns x SP parts, rounded up to whole waves.
-template <typename Tag, int DP, int NT>
+template <typename Tag, int DP, int SP, int NT>
 __global__ void __launch_bounds__(NT)
 hgrn2_scan_kernel(void* out, int64_t out_stride, const void* qpre, int64_t q_stride, const void* fpre, int64_t f_stride,
                   const void* v, int64_t v_stride, const float* f_bias, const float* lower, const float* norm_w, float* state,
                   int64_t state_stride, SeqBatch s, int H, int D, int Dv, float eps) {
   typedef Elem<Tag> E;
-  constexpr int kChunk = hgrn_chunk(DP), SP = hgrn_split(DP), DS = DP / SP, ROW = DP + 4 * SP;
+  constexpr int kChunk = hgrn_chunk(DP), DS = DP / SP, ROW = DP + 4 * SP;
   constexpr int PERK = (kChunk * DP + NT - 1) / NT;     // staged (token, query channel) elements per thread and pass
   constexpr int PERV = kChunk / SP;                     // value / output tokens per thread: tokens part + u SP of column col
   // (rows and parts start at multiples of 16 bytes: the token loop reads them four floats at a time)
@@ -151,20 +154,25 @@ static int launch_hgrn2(void* out, int64_t out_stride, const void* qpre, int64_t
                         float* state, int64_t state_stride, const SeqBatch& s, int H, int D, int Dv, float eps,
                         hipStream_t st) {
   const dim3 grid((unsigned)s.B, (unsigned)H);
-  if (Dv * (D > 64 ? 4 : (D > 32 ? 2 : 1)) > 1024) return SP_ERR_UNSUPPORTED;
   // (register rows past D take f = 0 and q = 0: whatever they hold never reaches an output and is never stored)
   // workgroup sizes come in steps (the staging's trip count is a compile-time number): the next one that holds Dv columns
-#define SP_HGRN_NT(DP, NT)                                                                                              \
-  hgrn2_scan_kernel<Tag, DP, NT><<<grid, NT, (size_t)hgrn_chunk(DP) * 2 * Dv * sizeof(float), st>>>(                    \
+#define SP_HGRN_NT(DP, SP, NT)                                                                                          \
+  hgrn2_scan_kernel<Tag, DP, SP, NT><<<grid, NT, (size_t)hgrn_chunk(DP) * 2 * Dv * sizeof(float), st>>>(                \
       out, out_stride, qpre, q_stride, fpre, f_stride, v, v_stride, f_bias, lower, norm_w, state, state_stride, s, H, D, Dv, eps)
+#define SP_HGRN_SP(DP, SP)                                                                                              \
+  do {                                                                                                                  \
+    const int need = Dv * SP;                                                                                           \
+    if (need <= 64) SP_HGRN_NT(DP, SP, 64);                                                                             \
+    else if (need <= 128) SP_HGRN_NT(DP, SP, 128);                                                                      \
+    else if (need <= 256) SP_HGRN_NT(DP, SP, 256);                                                                      \
+    else if (need <= 512) SP_HGRN_NT(DP, SP, 512);                                                                      \
+    else SP_HGRN_NT(DP, SP, 1024);                                                                                      \
+  } while (0)
 #define SP_HGRN(DP)                                                                                                     \
   do {                                                                                                                  \
-    const int need = Dv * hgrn_split(DP);                                                                               \
-    if (need <= 64) SP_HGRN_NT(DP, 64);                                                                                 \
-    else if (need <= 128) SP_HGRN_NT(DP, 128);                                                                          \
-    else if (need <= 256) SP_HGRN_NT(DP, 256);                                                                          \
-    else if (need <= 512) SP_HGRN_NT(DP, 512);                                                                          \
-    else SP_HGRN_NT(DP, 1024);                                                                                          \
+    if (Dv * hgrn_split_fine(DP) <= 1024) SP_HGRN_SP(DP, hgrn_split_fine(DP));                                          \
+    else if (Dv * hgrn_split_coarse(DP) <= 1024) SP_HGRN_SP(DP, hgrn_split_coarse(DP));                                 \
+    else return SP_ERR_UNSUPPORTED;                                                                                     \
   } while (0)
   if (D <= 16) SP_HGRN(16);
   else if (D <= 32) SP_HGRN(32);
@@ -173,6 +181,7 @@ static int launch_hgrn2(void* out, int64_t out_stride, const void* qpre, int64_t
   else if (D <= 256) SP_HGRN(256);
   else return SP_ERR_UNSUPPORTED;
 #undef SP_HGRN
+#undef SP_HGRN_SP
 #undef SP_HGRN_NT
   SP_LAUNCH_CHECK();
   return SP_OK;
