@@ -10,8 +10,9 @@
 //
 // One workgroup per (request, head): a column of S (one value channel) lives in the registers of 2, 4 or 8 neighbouring
 // lanes; the request's tokens of this step are walked in order from the state the previous step left in the pool (zeros
-// at a sequence's first token), staged through LDS in passes.  A token costs two sweeps over the column - u^T S first,
-// then the update with the numerator - and two lane exchanges, no workgroup barrier.  Prompt portions and single decoded
+// at a sequence's first token), staged through LDS in passes.  A token costs ONE sweep over the column: the update, the
+// numerator and - on the state just completed - the next token's u^T S, then two independent sums over the column's lanes
+// (register moves); no workgroup barrier.  Prompt portions and single decoded
 // tokens take the same path, and the order of every sum depends on the head only.
 #include "seq_batch.h"
 
@@ -90,7 +91,7 @@ delta_recurrence_kernel(void* out, int64_t out_stride, const void* r, int64_t r_
   constexpr int TSTEP = NT / KP, PER = kChunk / TSTEP;  // staging: thread j takes channel j % KP of tokens j / KP + u TSTEP
   constexpr int PERG = kChunk / SP;                     // epilogue: thread (col, part) takes tokens part + u SP
   // (rows and parts start at multiples of 16 bytes: the token loop reads them four floats at a time)
-  __shared__ __attribute__((aligned(16))) float sr[kChunk][ROW], sk[kChunk][ROW], sw[kChunk][ROW], su[kChunk][ROW], sau[kChunk][ROW];
+  __shared__ __attribute__((aligned(16))) float sr[kChunk][ROW], sk[kChunk][ROW], sw[kChunk][ROW], su[kChunk + 1][ROW], sau[kChunk][ROW];
   __shared__ float sv[kChunk][KP], so[kChunk][KP], sinv[kChunk];
   const int b = blockIdx.x, h = blockIdx.y, j = threadIdx.x;
   const int wave = j >> 6, lane = j & 63, waves = NT >> 6;
@@ -168,13 +169,11 @@ delta_recurrence_kernel(void* out, int64_t out_stride, const void* r, int64_t r_
     }
     __syncthreads();
     if (c0 + kChunk < len) fetch(c0 + kChunk);           // in flight while the recurrence runs
-    for (int tt = 0; tt < n; ++tt) {
-      const float4* pu = reinterpret_cast<const float4*>(&su[tt][mine]);
-      const float4* pau = reinterpret_cast<const float4*>(&sau[tt][mine]);
-      const float4* pw = reinterpret_cast<const float4*>(&sw[tt][mine]);
-      const float4* pk = reinterpret_cast<const float4*>(&sk[tt][mine]);
-      const float4* pr = reinterpret_cast<const float4*>(&sr[tt][mine]);
-      // (four partial sums per sweep: the chain of dependent additions is a quarter as long; DS is a multiple of 4)
+    // u^T S of the pass's first token; every later token's is formed in the sweep that completes the state it reads
+    // (four partial sums per sum: the chain of dependent additions is a quarter as long; DS is a multiple of 4)
+    float proj;
+    {
+      const float4* pu = reinterpret_cast<const float4*>(&su[0][mine]);
       float pj[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ii = 0; ii < DS; ii += 4) {
@@ -184,14 +183,19 @@ delta_recurrence_kernel(void* out, int64_t out_stride, const void* r, int64_t r_
         pj[2] += u4.z * S[ii + 2];
         pj[3] += u4.w * S[ii + 3];
       }
-      float proj = (pj[0] + pj[1]) + (pj[2] + pj[3]);
-#pragma unroll
-      for (int off = 1; off < SP; off <<= 1) proj += __shfl_xor(proj, off, 64);
+      proj = lanes_sum<SP>((pj[0] + pj[1]) + (pj[2] + pj[3]));
+    }
+    for (int tt = 0; tt < n; ++tt) {
+      const float4* pau = reinterpret_cast<const float4*>(&sau[tt][mine]);
+      const float4* pw = reinterpret_cast<const float4*>(&sw[tt][mine]);
+      const float4* pk = reinterpret_cast<const float4*>(&sk[tt][mine]);
+      const float4* pr = reinterpret_cast<const float4*>(&sr[tt][mine]);
+      const float4* pun = reinterpret_cast<const float4*>(&su[tt + 1][mine]);      // the next token's unit key (row n: unused)
       const float vj = live ? sv[tt][col] : 0.f;
-      float nm[4] = {0.f, 0.f, 0.f, 0.f};
+      float nm[4] = {0.f, 0.f, 0.f, 0.f}, pj[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ii = 0; ii < DS; ii += 4) {
-        const float4 w4 = pw[ii / 4], a4 = pau[ii / 4], k4 = pk[ii / 4], r4 = pr[ii / 4];
+        const float4 w4 = pw[ii / 4], a4 = pau[ii / 4], k4 = pk[ii / 4], r4 = pr[ii / 4], u4 = pun[ii / 4];
         S[ii] = w4.x * S[ii] - a4.x * proj + k4.x * vj;
         S[ii + 1] = w4.y * S[ii + 1] - a4.y * proj + k4.y * vj;
         S[ii + 2] = w4.z * S[ii + 2] - a4.z * proj + k4.z * vj;
@@ -200,10 +204,13 @@ delta_recurrence_kernel(void* out, int64_t out_stride, const void* r, int64_t r_
         nm[1] += S[ii + 1] * r4.y;
         nm[2] += S[ii + 2] * r4.z;
         nm[3] += S[ii + 3] * r4.w;
+        pj[0] += S[ii] * u4.x;
+        pj[1] += S[ii + 1] * u4.y;
+        pj[2] += S[ii + 2] * u4.z;
+        pj[3] += S[ii + 3] * u4.w;
       }
-      float num = (nm[0] + nm[1]) + (nm[2] + nm[3]);
-#pragma unroll
-      for (int off = 1; off < SP; off <<= 1) num += __shfl_xor(num, off, 64);
+      const float num = lanes_sum<SP>((nm[0] + nm[1]) + (nm[2] + nm[3]));
+      proj = lanes_sum<SP>((pj[0] + pj[1]) + (pj[2] + pj[3]));
       if (live && part == 0) so[tt][col] = num;
     }
     __syncthreads();

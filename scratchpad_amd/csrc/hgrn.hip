@@ -118,9 +118,7 @@ hgrn2_scan_kernel(void* out, int64_t out_stride, const void* qpre, int64_t q_str
         nm[2] += S[ii + 2] * q4.z;
         nm[3] += S[ii + 3] * q4.w;
       }
-      float num = (nm[0] + nm[1]) + (nm[2] + nm[3]);
-#pragma unroll
-      for (int off = 1; off < SP; off <<= 1) num += __shfl_xor(num, off, 64);
+      const float num = lanes_sum<SP>((nm[0] + nm[1]) + (nm[2] + nm[3]));
       if (live && part == 0) so[tt * Dv + col] = num;
     }
     __syncthreads();

@@ -198,6 +198,21 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// sum over N neighbouring lanes (aligned groups of N = 1, 2, 4 or 8) by data-parallel-primitive moves - register-to-register,
+// no trip through the LDS crossbar that __shfl_xor takes; every lane of a group ends with the same value
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+template <int N>
+__device__ __forceinline__ float lanes_sum(float v) {
+  static_assert(N == 1 || N == 2 || N == 4 || N == 8, "lanes per group");
+  if constexpr (N >= 2) v += dpp_f32<0xB1>(v);      // quad_perm [1,0,3,2]: lane ^ 1
+  if constexpr (N >= 4) v += dpp_f32<0x4E>(v);      // quad_perm [2,3,0,1]: lane ^ 2
+  if constexpr (N >= 8) v += dpp_f32<0x141>(v);     // row_half_mirror: lane i <-> 7 - i of each 8 (the other quad's sum)
+  return v;
+}
+
 // index arrays that are int64 in eager mode and int32 under graph replay
 __device__ __forceinline__ int64_t load_idx(const void* p, int i, int idx64) {
   return idx64 ? ((const int64_t*)p)[i] : (int64_t)((const int32_t*)p)[i];
