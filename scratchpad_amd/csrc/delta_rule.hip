@@ -70,8 +70,9 @@ delta_gates_kernel(float* decay, float* remove, const void* p, int64_t p_stride,
 
 constexpr int delta_chunk(int KP) { return KP > 64 ? 8 : 16; }                      // tokens staged in LDS per pass
 // lanes that share one column of S: 8 state values per lane where the workgroup's 1024 threads allow it (measured at heads of
-// 64: 2 lanes 1.07 ms, 4 lanes 0.58 ms, 8 lanes 0.38 ms, 16 lanes 0.49 ms per 4096 tokens - more waves per SIMD hide the
-// waits of the per-token chain until the lane exchanges take over)
+// 64: 2 lanes 1.07 ms, 4 lanes 0.58 ms, 8 lanes 0.38 ms, 16 lanes 0.49 ms per 4096 tokens with two sweeps per token and
+// lane exchanges through LDS; 8 lanes 0.29 ms, 16 lanes 0.32 ms with one sweep and register moves - more waves per SIMD
+// hide the waits of the per-token chain until the sums over the lanes take over)
 constexpr int delta_split(int KP) { return KP > 128 ? 4 : (KP > 32 ? 8 : (KP > 16 ? 4 : 2)); }
 
 // thread = (column col of S, part): part p of SP owns the rows [p DS, (p + 1) DS) of the column.  LDS rows are padded by
