@@ -69,7 +69,7 @@ def toredra_config(width: int, layers: int, context_len: int):
     dense = {"kind": "dense", "ff": {2048: 8192, 4096: 14336}.get(width, 3 * width)}
     pattern = [delta, delta, par, delta]
     raw = {"architecture": "Toredra", "vocab": 128256, "width": width, "norm": {"eps": 1e-5}, "logit_scale": 0.5,
-           "logit_softcap": 30.0, "layers": [{**pattern[i % 4], "mlp": dense} for i in range(layers)]}
+           "logit_softcap": 50.0, "layers": [{**pattern[i % 4], "mlp": dense} for i in range(layers)]}
     return ToredraConfig(raw, context_len=context_len, decay_rank=64)
 
 

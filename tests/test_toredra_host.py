@@ -71,7 +71,7 @@ def test_sink_only_shrinks_the_output():
 
 def test_frequency_rule_of_oracle_and_product_agree():
     from scratchpad_amd.layers import AngleRotary, wavelength_blend
-    for rot in ({"dims": 48, "base": 50000.0, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 512}},
+    for rot in ({"dims": 40, "base": 30000.0, "scaling": {"factor": 8.0, "low": 1.0, "high": 3.0, "original": 512}},
                 {"dims": 16, "base": 100.0, "scaling": {"factor": 3.0, "low": 2.0, "high": 2.0, "original": 40}},
                 {"dims": 8, "base": 10000.0}):
         f = to.rotary_frequencies(rot)

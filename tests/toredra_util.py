@@ -86,4 +86,4 @@ def random_config(seed: int):
         a = r.randint(0, n - 1)
         loop = (a, r.randint(a + 1, n), r.choice([1, 2, 3]))
     return config(layers, width=r.choice([48, 64, 96, 128]), vocab=r.choice([61, 130, 257]), eps=r.choice([1e-6, 1e-5]),
-                  loop=loop, logit_scale=r.choice([None, 0.25, 2.0]), softcap=r.choice([None, 5.0, 30.0]))
+                  loop=loop, logit_scale=r.choice([None, 0.3, 2.0]), softcap=r.choice([None, 5.0, 25.0]))
