@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define SP_ABI_VERSION 12
+#define SP_ABI_VERSION 13
 #define SP_API __attribute__((visibility("default")))
 
 typedef enum { SP_F32 = 0, SP_F16 = 1, SP_BF16 = 2, SP_FP8_E5M2 = 3 /* KV pool only */ } sp_dtype;
@@ -484,8 +484,9 @@ SP_API int sp_moe_combine(void* out, const void* z, const int32_t* place, const 
 /* Choice of experts by softmax scores on ready fp32 logits [T, experts] (sp_small_linear_f32 makes them): s = softmax
  * over all experts; ids [T, top] = the experts with the largest s (ties: the lower index), weights [T, top] = their s
  * times scale, not renormalised.                                                                                    */
+/* renorm != 0 (ABI 13): the weights are divided by their sum - the softmax over the chosen logits only.              */
 SP_API int sp_moe_softmax_topk(int32_t* ids, float* weights, const float* logits, int64_t num_tokens, int experts, int top,
-                               float scale, void* stream);
+                               float scale, int renorm, void* stream);
 
 /* ---- fp32 residual stream of parallel-sublayer layers (csrc/stream_norm.hip) ------------------------------------- */
 /* x[t] = embed[ids[t]] * scale  (x fp32, embed in `dtype`) */
@@ -514,7 +515,13 @@ SP_API int sp_qkv_rotary_store(void* q, int64_t q_stride, const void* k, int64_t
                                void* kpool, int64_t kp_stride, void* vpool, int64_t vp_stride, const int64_t* positions,
                                const int64_t* loc, const float* freq, float mag, const float* q_bias, const float* k_bias,
                                const float* v_bias, int64_t num_tokens, int heads, int kv_heads, int dim, int vdim,
-                               int rot_dims, int adjacent, int norm_values, float eps, int dtype, void* stream);
+                               int rot_dims, int adjacent, int norm_values, float eps, int qk_norm, const float* q_head_scale,
+                               float q_temp_coef, int q_temp_every, const void* v_first, int64_t vf_stride,
+                               const float* v_mix, int dtype, void* stream);
+/* (ABI 13) qk_norm != 0: q and k are divided per head by their root mean square over dim after the rotation (eps inside
+ * the root).  q_head_scale (fp32 [heads], optional) and, with q_temp_every > 0, 1 + q_temp_coef * ln(floor((position + 1) /
+ * q_temp_every) + 1) multiply q afterwards.  v_first (a pool of vpool's shape and type, row stride vf_stride; optional):
+ * the stored value is (1 - v_mix[0]) v + v_mix[0] v_first[loc[t]].  These forms need dim, vdim <= 256.                    */
 /* every token of the step whose position + 1 is a multiple of `block` writes the mean of the last `block` cached key rows
  * (value rows) of its request into kpooled (vpooled) at its own slot; run after the step's rows are in the pool       */
 SP_API int sp_pool_blocks(void* kpooled, void* vpooled, const void* kpool, const void* vpool, int64_t kp_stride,
@@ -531,7 +538,11 @@ SP_API int sp_window_attention(void* out, int64_t out_stride, const void* q, int
                                const void* vpool, const void* kpooled, const void* vpooled, int64_t kp_stride,
                                int64_t vp_stride, const int32_t* req_to_token, int64_t table_stride, int64_t num_tokens,
                                int heads, int kv_heads, int dim, int vdim, int64_t window, int block, float scale,
-                               const float* sinks, int matrix, SP_SEQ_PARAMS, int dtype, void* stream);
+                               const float* sinks, float softcap, int sigmoid_weights, const float* head_bias,
+                               const void* gate, int64_t gate_stride, int matrix, SP_SEQ_PARAMS, int dtype, void* stream);
+/* (ABI 13) softcap > 0: score = softcap tanh(score / softcap) after the scale.  sigmoid_weights != 0: no softmax - a
+ * visible key's weight is sigmoid(score + head_bias[head]) (head_bias fp32 [heads], optional), not normalised; no sinks.
+ * gate ([T, heads * vdim] in `dtype`, optional): the result is multiplied element by element with sigmoid(gate).        */
 
 /* ---- state-space and matrix-memory recurrences (csrc/ssm.hip, csrc/mlstm.hip) -------------------------------------- */
 /* out[t, j] = bias[j] + sum_i weight[j, i] x[t, i]: fp32 weights, accumulation and output (x in `dtype`; bias optional) */
@@ -610,6 +621,33 @@ SP_API int sp_hgrn2_scan(void* out, int64_t out_stride, const void* qpre, int64_
                          int64_t f_stride, const void* v, int64_t v_stride, const float* f_bias, const float* lower,
                          const float* norm_w, float* state, int64_t state_stride, int heads, int dim, int vdim, float eps,
                          SP_SEQ_PARAMS, int dtype, void* stream);
+
+
+/* ================================================================================================================
+ * ABI 13: a norm in groups on the fp32 stream, the channel-gated delta rule and its low-rank gates.
+ */
+/* x = x + a, or x + (N(a) wa + N(b) wb) / 2 with a second branch (N = division by the row's root mean square), or x as it
+ * is (a null); out_next (optional, in `dtype`) = GN(x) next_weight, GN = each of `groups` equal consecutive parts of the
+ * row divided by its own root mean square (eps inside the root).  x fp32 in place; a, b in `dtype`.                    */
+SP_API int sp_add_group_norm(float* x, int64_t x_stride, const void* a, int64_t a_stride, const float* wa, const void* b,
+                             int64_t b_stride, const float* wb, void* out_next, int64_t next_stride, const float* next_weight,
+                             int64_t num_tokens, int width, int groups, float eps, int dtype, void* stream);
+/* out fp32 [T, channels]: z = sum_r w2t[r, c] p[t, r] + bias[c] (p [T, rank] in `dtype`, w2t fp32 [rank, channels], bias
+ * optional); act 0: exp(-exp(A_log[c / per_head]) softplus(z)), act 1: sigmoid(z).                                      */
+SP_API int sp_lowrank_gate(float* out, const void* p, int64_t p_stride, const float* w2t, const float* bias,
+                           const float* A_log, int64_t num_tokens, int channels, int rank, int per_head, int act, int dtype,
+                           void* stream);
+/* Per (request, value head h) over the request's rows of this step in order, S [dim, vdim] fp32 from state[request slot]
+ * (zeros at a sequence's first token) and back; query/key head h / (heads / kv_heads):
+ *   qn = q / sqrt(|q|^2 + 1e-6) dim^(-1/2);  kn = k / sqrt(|k|^2 + 1e-6);  S = diag(decay) S;
+ *   u = sigmoid(bpre) (v - S^T kn);  S = S + kn u^T;  o = S^T qn;  out = o / rms_head(o) * norm_w * gate
+ * q, k [T, kv_heads * dim], v, out [T, heads * vdim], bpre [T, heads] in `dtype`; decay fp32 [T, heads * dim], gate fp32
+ * [T, heads * vdim], norm_w fp32 [vdim].  dim, vdim <= 256.                                                             */
+SP_API int sp_gated_delta_scan(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k,
+                               int64_t k_stride, const void* v, int64_t v_stride, const void* bpre, int64_t b_stride,
+                               const float* decay, const float* gate, const float* norm_w, float* state,
+                               int64_t state_stride, int heads, int kv_heads, int dim, int vdim, float eps, SP_SEQ_PARAMS,
+                               int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -8,7 +8,7 @@ signalled, managers/tp_worker_client.py:110-116).  Tensors are passed as raw dev
 import ctypes
 import os
 import weakref
-from typing import Optional
+from typing import Optional, Tuple
 
 import torch
 
@@ -125,16 +125,17 @@ SIGNATURES = {
     "sp_moe_glu": (_i32, [_vp, _vp, _i64, _i32, _f32, _f32, _i32, _vp]),
     "sp_moe_combine": (_i32, [_vp, _vp, _vp, _vp, _i64, _i32, _i32, _i64, _i32, _vp]),
     # ---- ABI 11
-    "sp_moe_softmax_topk": (_i32, [_vp, _vp, _vp, _i64, _i32, _i32, _f32, _vp]),
+    "sp_moe_softmax_topk": (_i32, [_vp, _vp, _vp, _i64, _i32, _i32, _f32, _i32, _vp]),
     "sp_embed_scale": (_i32, [_vp, _i64, _vp, _vp, _i64, _i32, _i64, _f32, _i32, _vp]),
     "sp_norm_shift": (_i32, [_vp, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i32, _f32, *_SEQ, _i32, _vp]),
     "sp_norm_save_last": (_i32, [_vp, _i64, _vp, _i64, _vp, _i32, _f32, *_SEQ, _vp]),
     "sp_stream_add": (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _i64, _i32, _i32, _vp]),
     "sp_qkv_rotary_store": (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _f32, _vp, _vp, _vp,
-                                   _i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _vp]),
+                                   _i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _vp, _f32, _i32, _vp, _i64, _vp,
+                                   _i32, _vp]),
     "sp_pool_blocks": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i32, _i32, _i32, *_SEQ, _i32, _vp]),
     "sp_window_attention": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _i32, _i32, _i32,
-                                   _i32, _i64, _i32, _f32, _vp, _i32, *_SEQ, _i32, _vp]),
+                                   _i32, _i64, _i32, _f32, _vp, _f32, _i32, _vp, _vp, _i64, _i32, *_SEQ, _i32, _vp]),
     "sp_small_linear_f32": (_i32, [_vp, _vp, _i64, _vp, _vp, _i64, _i32, _i32, _i32, _vp]),
     "sp_causal_conv_silu": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i32, _i32, *_SEQ, _i32, _vp]),
     "sp_mamba2_scan": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, *_SEQ, _i32, _vp]),
@@ -151,6 +152,11 @@ SIGNATURES = {
                                    _f32, *_SEQ, _i32, _vp]),
     "sp_hgrn2_scan": (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _f32,
                              *_SEQ, _i32, _vp]),
+    # ---- ABI 13
+    "sp_add_group_norm": (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _i64, _vp, _vp, _i64, _vp, _i64, _i32, _i32, _f32, _i32, _vp]),
+    "sp_lowrank_gate": (_i32, [_vp, _vp, _i64, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32, _vp]),
+    "sp_gated_delta_scan": (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _i32, _i32,
+                                   _i32, _i32, _f32, *_SEQ, _i32, _vp]),
 }
 
 
@@ -184,7 +190,7 @@ def load() -> ctypes.CDLL:
             continue
         fn.restype = res
         fn.argtypes = args
-    if lib.sp_abi_version() != 12:
+    if lib.sp_abi_version() != 13:
         raise RuntimeError("libscratchpad_hip.so ABI version mismatch")
     _lib = lib
     return lib
@@ -1202,14 +1208,16 @@ def moe_combine(z: torch.Tensor, place: torch.Tensor, weights: torch.Tensor) -> 
 
 
 # --------------------------------------------------------------------------- fp32 stream with token shift, windowed attention, scans
-def moe_route_softmax(x: torch.Tensor, router: torch.Tensor, top: int, scale: float):
-    """(ids int32 [T, top], weights fp32 [T, top]): fp32 logits router x, the largest softmax scores, times scale"""
-    logits = small_linear_f32(x, router)
+def moe_route_softmax(x: torch.Tensor, router: torch.Tensor, top: int, scale: float, bias: Optional[torch.Tensor] = None,
+                      renorm: bool = False):
+    """(ids int32 [T, top], weights fp32 [T, top]): fp32 logits router x (+ bias), the largest softmax scores, times scale;
+    ``renorm``: divided by their sum (the softmax over the chosen logits only)"""
+    logits = small_linear_f32(x, router, bias)
     T, E = logits.shape
     ids = torch.empty((T, top), dtype=torch.int32, device=x.device)
     weights = torch.empty((T, top), dtype=torch.float32, device=x.device)
-    _check(load().sp_moe_softmax_topk(ids.data_ptr(), weights.data_ptr(), logits.data_ptr(), T, E, top, scale, _stream()),
-           "sp_moe_softmax_topk")
+    _check(load().sp_moe_softmax_topk(ids.data_ptr(), weights.data_ptr(), logits.data_ptr(), T, E, top, scale, int(renorm),
+                                      _stream()), "sp_moe_softmax_topk")
     return ids, weights
 
 
@@ -1267,10 +1275,15 @@ def qkv_rotary_store(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, kpool: t
                      positions: torch.Tensor, loc: torch.Tensor, freq: Optional[torch.Tensor], mag: float, heads: int,
                      kv_heads: int, dim: int, vdim: int, eps: float, adjacent: bool = False, norm_values: bool = True,
                      q_bias: Optional[torch.Tensor] = None, k_bias: Optional[torch.Tensor] = None,
-                     v_bias: Optional[torch.Tensor] = None) -> None:
+                     v_bias: Optional[torch.Tensor] = None, qk_norm: bool = False, q_head_scale: Optional[torch.Tensor] = None,
+                     q_temp: Optional[Tuple[float, int]] = None, v_first: Optional[torch.Tensor] = None,
+                     v_mix: Optional[torch.Tensor] = None) -> None:
     """q [T, heads * dim] rotated in place; k rotated, v (head-normed unless ``norm_values`` is off) into the pools' rows
     loc (views: strides are taken).  ``adjacent``: coordinate 2i pairs with 2i + 1 instead of i with i + dims / 2.  fp32
-    biases, where given, are added before the rotation / the norm."""
+    biases, where given, are added before the rotation / the norm.  ``qk_norm``: q and k divided per head by their root
+    mean square after the rotation; ``q_head_scale`` fp32 [heads] and ``q_temp`` = (coef, every): q times the head's number
+    and times 1 + coef ln(floor((position + 1) / every) + 1); ``v_first`` (another layer's value pool) with ``v_mix`` (fp32,
+    one number): the stored value is (1 - v_mix) v + v_mix v_first[loc]."""
     for name, t, n in (("q", q, heads * dim), ("k", k, kv_heads * dim), ("v", v, kv_heads * vdim)):
         if _mat(t, name).shape[1] != n or t.dtype != q.dtype or t.shape[0] != q.shape[0]:
             raise RuntimeError(f"qkv_rotary_store: {name} must be [T, {n}]")
@@ -1283,11 +1296,19 @@ def qkv_rotary_store(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, kpool: t
         if t is not None and _f32(t, name).numel() != n:
             raise RuntimeError(f"qkv_rotary_store: {name} must hold {n} values")
     dims = 0 if freq is None else 2 * _f32(freq, "freq").shape[0]
+    if q_head_scale is not None and _f32(q_head_scale, "q_head_scale").numel() != heads:
+        raise RuntimeError("qkv_rotary_store: q_head_scale must hold one value per query head")
+    if v_first is not None and (v_mix is None or _f32(v_mix, "v_mix").numel() != 1 or v_first.shape != vpool.shape or
+                                v_first.dtype != vpool.dtype):
+        raise RuntimeError("qkv_rotary_store: v_first must mirror vpool and come with v_mix (one fp32 number)")
+    coef, every = q_temp if q_temp else (0.0, 0)
     _check(load().sp_qkv_rotary_store(q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
                                       kpool.data_ptr(), kpool.stride(0), vpool.data_ptr(), vpool.stride(0), positions.data_ptr(),
                                       loc.data_ptr(), _ptr(freq), mag, _ptr(q_bias), _ptr(k_bias), _ptr(v_bias), q.shape[0],
-                                      heads, kv_heads, dim, vdim, dims, int(adjacent), int(norm_values), eps, _dt(q),
-                                      _stream()), "sp_qkv_rotary_store")
+                                      heads, kv_heads, dim, vdim, dims, int(adjacent), int(norm_values), eps, int(qk_norm),
+                                      _ptr(q_head_scale), float(coef), int(every), _ptr(v_first),
+                                      0 if v_first is None else v_first.stride(0), _ptr(v_mix), _dt(q), _stream()),
+           "sp_qkv_rotary_store")
 
 
 def pool_blocks(kpooled: torch.Tensor, vpooled: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor,
@@ -1303,9 +1324,12 @@ def pool_blocks(kpooled: torch.Tensor, vpooled: torch.Tensor, kpool: torch.Tenso
 def window_attention(q: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, kpooled: Optional[torch.Tensor],
                      vpooled: Optional[torch.Tensor], req_to_token: torch.Tensor, seq: SeqParams, heads: int, kv_heads: int,
                      dim: int, vdim: int, window: int, block: int, scale: float, matrix: bool = True,
-                     sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     sinks: Optional[torch.Tensor] = None, softcap: float = 0.0, sigmoid_weights: bool = False,
+                     head_bias: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """q [T, heads * dim] (rotated) -> [T, heads * vdim]; matrix=False keeps 16-bit prompt portions off the matrix-core
-    kernel (comparisons); sinks fp32 [heads]: one more term exp(sink) in every softmax's denominator"""
+    kernel (comparisons); sinks fp32 [heads]: one more term exp(sink) in every softmax's denominator; softcap > 0: scores
+    capped as softcap tanh(score / softcap); sigmoid_weights: a visible key's weight is sigmoid(score + head_bias[head]),
+    not normalised; gate [T, heads * vdim] (a view): the result times sigmoid(gate)"""
     _mat(q, "q"), _mat(kpool, "kpool"), _mat(vpool, "vpool")
     T = q.shape[0]
     if q.shape[1] != heads * dim or kpool.shape[1] != kv_heads * dim or vpool.shape[1] != kv_heads * vdim or \
@@ -1315,11 +1339,17 @@ def window_attention(q: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, 
         raise RuntimeError("window_attention: pooled buffers must mirror the token buffers")
     if sinks is not None and _f32(sinks, "sinks").numel() != heads:
         raise RuntimeError("window_attention: sinks must hold one value per query head")
+    if head_bias is not None and _f32(head_bias, "head_bias").numel() != heads:
+        raise RuntimeError("window_attention: head_bias must hold one value per query head")
+    if gate is not None and (_mat(gate, "gate").shape != (T, heads * vdim) or gate.dtype != q.dtype):
+        raise RuntimeError("window_attention: gate must be [T, heads * vdim] of q's dtype")
     out = empty_rows(T, heads * vdim, q.dtype, q.device)
     _check(load().sp_window_attention(out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), kpool.data_ptr(),
                                       vpool.data_ptr(), _ptr(kpooled), _ptr(vpooled), kpool.stride(0), vpool.stride(0),
                                       req_to_token.data_ptr(), req_to_token.stride(0), T, heads, kv_heads, dim, vdim,
-                                      window, block, scale, _ptr(sinks), int(matrix), *seq.args, _dt(q), _stream()),
+                                      window, block, scale, _ptr(sinks), float(softcap or 0.0), int(sigmoid_weights),
+                                      _ptr(head_bias), _ptr(gate), 0 if gate is None else gate.stride(0), int(matrix),
+                                      *seq.args, _dt(q), _stream()),
            "sp_window_attention")
     return out
 
@@ -1505,4 +1535,73 @@ def hgrn2_scan(qpre: torch.Tensor, fpre: torch.Tensor, v: torch.Tensor, f_bias: 
                                 v.data_ptr(), v.stride(0), f_bias.data_ptr(), lower.data_ptr(), norm_w.data_ptr(),
                                 state.data_ptr(), state.stride(0), heads, dim, vdim, eps, *seq.args, _dt(qpre), _stream()),
            "sp_hgrn2_scan")
+    return out
+
+
+# --------------------------------------------------------------------------- norm in groups, channel-gated delta rule
+def add_group_norm(x: torch.Tensor, a: Optional[torch.Tensor], groups: int, eps: float, dtype: torch.dtype,
+                   b: Optional[torch.Tensor] = None, wa: Optional[torch.Tensor] = None, wb: Optional[torch.Tensor] = None,
+                   next_weight: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """x fp32 [T, W] += a (or (N(a) wa + N(b) wb) / 2 with a second branch; nothing when a is None) in place; with
+    ``next_weight`` returns GN(x) * next_weight in ``dtype``: every one of ``groups`` equal parts of the row divided by its
+    own root mean square.  a, b may be views (their row strides are taken)."""
+    _mat(x, "x")
+    T, W = x.shape
+    if x.dtype != torch.float32 or W % groups:
+        raise RuntimeError("add_group_norm: x fp32 [T, W], W divisible by groups")
+    for name, t in (("a", a), ("b", b)):
+        if t is not None and (_mat(t, name).shape != (T, W) or t.dtype != dtype):
+            raise RuntimeError(f"add_group_norm: {name} must be [T, W] of the given dtype")
+    if b is not None and (a is None or wa is None or wb is None or _f32(wa, "wa").numel() != W or _f32(wb, "wb").numel() != W):
+        raise RuntimeError("add_group_norm: two branches need their norm weights wa, wb [W]")
+    nxt = None
+    if next_weight is not None:
+        if _f32(next_weight, "next_weight").numel() != W:
+            raise RuntimeError("add_group_norm: next_weight [W]")
+        nxt = empty_rows(T, W, dtype, x.device)
+    elif a is None:
+        return None
+    _check(load().sp_add_group_norm(x.data_ptr(), x.stride(0), _ptr(a), 0 if a is None else a.stride(0), _ptr(wa), _ptr(b),
+                                    0 if b is None else b.stride(0), _ptr(wb), _ptr(nxt), 0 if nxt is None else nxt.stride(0),
+                                    _ptr(next_weight), T, W, groups, eps, _DTYPES[dtype], _stream()), "sp_add_group_norm")
+    return nxt
+
+
+def lowrank_gate(p: torch.Tensor, w2t: torch.Tensor, bias: Optional[torch.Tensor], act: str,
+                 A_log: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp32 [T, channels]: z = p w2t + bias (p [T, rank] a view, w2t fp32 [rank, channels]); act "decay":
+    exp(-exp(A_log[head]) softplus(z)) with channels / len(A_log) channels per head, act "sigmoid": sigmoid(z)"""
+    _mat(p, "p"), _f32(w2t, "w2t")
+    T, (rank, n) = p.shape[0], w2t.shape
+    if p.shape[1] != rank or (bias is not None and _f32(bias, "bias").numel() != n) or act not in ("decay", "sigmoid"):
+        raise RuntimeError("lowrank_gate: p [T, rank], w2t [rank, channels], bias [channels]")
+    per = 1
+    if act == "decay":
+        if A_log is None or n % _f32(A_log, "A_log").numel():
+            raise RuntimeError("lowrank_gate: the decay needs A_log [heads], heads dividing the channels")
+        per = n // A_log.numel()
+    out = torch.empty((T, n), dtype=torch.float32, device=p.device)
+    _check(load().sp_lowrank_gate(out.data_ptr(), p.data_ptr(), p.stride(0), w2t.data_ptr(), _ptr(bias), _ptr(A_log), T, n, rank,
+                                  per, 0 if act == "decay" else 1, _dt(p), _stream()), "sp_lowrank_gate")
+    return out
+
+
+def gated_delta_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, bpre: torch.Tensor, decay: torch.Tensor,
+                     gate: torch.Tensor, norm_w: torch.Tensor, state: torch.Tensor, seq: SeqParams, heads: int, kv_heads: int,
+                     dim: int, vdim: int, eps: float) -> torch.Tensor:
+    """q, k [T, kv_heads * dim], v [T, heads * vdim], bpre [T, heads] (views) -> [T, heads * vdim]; decay fp32
+    [T, heads * dim], gate fp32 [T, heads * vdim]; state [slots, heads, dim, vdim] fp32 is read and moved on"""
+    T = seq.num_tokens
+    for name, t, w in (("q", q, kv_heads * dim), ("k", k, kv_heads * dim), ("v", v, heads * vdim), ("bpre", bpre, heads)):
+        if _mat(t, name).shape != (T, w) or t.dtype != q.dtype:
+            raise RuntimeError(f"gated_delta_scan: {name} must be [num_tokens, {w}] of one dtype")
+    _f32(decay, "decay"), _f32(gate, "gate"), _f32(norm_w, "norm_w"), _f32(state, "state")
+    if decay.shape != (T, heads * dim) or gate.shape != (T, heads * vdim) or norm_w.numel() != vdim or \
+            state.shape[1:] != (heads, dim, vdim) or not decay.is_contiguous() or not gate.is_contiguous():
+        raise RuntimeError("gated_delta_scan: decay [T, H*D], gate [T, H*Dv], norm_w [Dv], state [slots, H, D, Dv]")
+    out = empty_rows(T, heads * vdim, q.dtype, q.device)
+    _check(load().sp_gated_delta_scan(out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0),
+                                      v.data_ptr(), v.stride(0), bpre.data_ptr(), bpre.stride(0), decay.data_ptr(),
+                                      gate.data_ptr(), norm_w.data_ptr(), state.data_ptr(), state.stride(0), heads, kv_heads,
+                                      dim, vdim, eps, *seq.args, _dt(q), _stream()), "sp_gated_delta_scan")
     return out

@@ -539,10 +539,18 @@ class PooledWindowAttention(nn.Module):
     softmax over both); key width ``dim`` and value width ``vdim`` may differ.  window None: plain causal attention.
     ``sinks``: one learned fp32 number per query head whose exponential joins the softmax's denominator (a key every query
     sees, without a value).  ``norm_values``: the cache holds every value head divided by its root mean square.  q, k, v may
-    carry fp32 biases (``store``), added before the rotation."""
+    carry fp32 biases (``store``), added before the rotation.
+    ``qk_norm``: q and k are divided per head by their root mean square after the rotation.  ``head_scale``: a learned fp32
+    number per query head that multiplies its scores (folded into q).  ``q_temp`` = (coef, every): q of position p times
+    1 + coef ln(floor((p + 1) / every) + 1).  ``softcap``: scores capped as cap tanh(score / cap).  ``weights`` = "sigmoid":
+    no softmax - a visible key weighs sigmoid(score + head_bias[head]) (``head_bias`` a learned fp32 number per head), not
+    normalised.  ``v_mix``: the cached value is (1 - v_mix) v + v_mix v_first, v_first being what the pool layer named at
+    ``store`` holds for the same token (v_mix a learned fp32 number)."""
 
     def __init__(self, num_heads: int, num_kv_heads: int, dim: int, vdim: int, scaling: float, layer_id: int,
-                 window: Optional[int] = None, block: Optional[int] = None, sinks: bool = False, norm_values: bool = True):
+                 window: Optional[int] = None, block: Optional[int] = None, sinks: bool = False, norm_values: bool = True,
+                 qk_norm: bool = False, head_scale: bool = False, q_temp=None, softcap: float = 0.0,
+                 weights: str = "softmax", v_mix: bool = False):
         super().__init__()
         if num_heads % num_kv_heads:
             raise ValueError("query heads must be a multiple of key/value heads")
@@ -551,18 +559,29 @@ class PooledWindowAttention(nn.Module):
         self.window = int(window) if window else 0
         self.block = int(block) if (block and window) else 0
         self.norm_values = norm_values
-        self.sinks = nn.Parameter(torch.zeros(num_heads, dtype=torch.float32), requires_grad=False) if sinks else None
+        if weights not in ("softmax", "sigmoid") or (weights == "sigmoid" and sinks):
+            raise ValueError("weights: 'softmax' or 'sigmoid' (which has no sink)")
+        f32 = dict(dtype=torch.float32)
+        self.sinks = nn.Parameter(torch.zeros(num_heads, **f32), requires_grad=False) if sinks else None
+        self.qk_norm, self.softcap, self.sigmoid_weights = qk_norm, float(softcap or 0.0), weights == "sigmoid"
+        self.q_temp = (float(q_temp[0]), int(q_temp[1])) if q_temp else None
+        self.head_scale = nn.Parameter(torch.ones(num_heads, **f32), requires_grad=False) if head_scale else None
+        self.head_bias = nn.Parameter(torch.zeros(num_heads, **f32), requires_grad=False) if self.sigmoid_weights else None
+        self.v_mix = nn.Parameter(torch.zeros(1, **f32), requires_grad=False) if v_mix else None
 
     def store(self, q, k, v, rotary, positions, eps: float, forward_batch: "ForwardBatch", cache_id: Optional[int] = None,
-              biases=(None, None, None)) -> None:
+              biases=(None, None, None), v_first_cache: Optional[int] = None) -> None:
         """rotate q in place; rotate k, norm v per head (if the layer does) and put both into the pool; then the blocks this
         step completes.  ``cache_id``: the pool layer to use instead of ``layer_id`` (a layer that runs several times on the
-        same weights keeps one cache per run)."""
-        forward_batch.attn_backend.store_window(q, k, v, rotary, positions, eps, self, forward_batch, cache_id, biases)
+        same weights keeps one cache per run).  ``v_first_cache``: the pool layer whose values this layer's are blended
+        with (a layer built with ``v_mix``; None: no blending, the layer is the one others blend with)."""
+        forward_batch.attn_backend.store_window(q, k, v, rotary, positions, eps, self, forward_batch, cache_id, biases,
+                                                v_first_cache)
 
-    def forward(self, q, forward_batch: "ForwardBatch", cache_id: Optional[int] = None):
-        """q [T, heads * dim] (rotated) -> [T, heads * vdim]; the step's rows are in the pool"""
-        return forward_batch.attn_backend.forward_window(q, self, forward_batch, cache_id)
+    def forward(self, q, forward_batch: "ForwardBatch", cache_id: Optional[int] = None, gate=None):
+        """q [T, heads * dim] (rotated) -> [T, heads * vdim]; the step's rows are in the pool.  ``gate`` [T, heads * vdim]:
+        the result times sigmoid(gate)"""
+        return forward_batch.attn_backend.forward_window(q, self, forward_batch, cache_id, gate)
 
 
 class SequenceBackend(AttentionBackend):
@@ -608,7 +627,7 @@ class SequenceBackend(AttentionBackend):
                                         layer.scaling)
 
     def store_window(self, q, k, v, rotary, positions, eps, layer: "PooledWindowAttention", forward_batch: "ForwardBatch",
-                     cache_id=None, biases=(None, None, None)):
+                     cache_id=None, biases=(None, None, None), v_first_cache=None):
         pool = forward_batch.token_to_kv_pool
         cache = layer.layer_id if cache_id is None else cache_id
         kbuf, vbuf = pool.get_kv_buffer(cache)
@@ -616,12 +635,15 @@ class SequenceBackend(AttentionBackend):
         _native.qkv_rotary_store(q, k, v, kbuf, vbuf, positions, forward_batch.out_cache_loc, freq, mag, layer.tp_q_head_num,
                                  layer.tp_k_head_num, layer.dim, layer.vdim, eps,
                                  adjacent=bool(rotary is not None and rotary.adjacent_pairs), norm_values=layer.norm_values,
-                                 q_bias=biases[0], k_bias=biases[1], v_bias=biases[2])
+                                 q_bias=biases[0], k_bias=biases[1], v_bias=biases[2], qk_norm=layer.qk_norm,
+                                 q_head_scale=None if layer.head_scale is None else layer.head_scale.data, q_temp=layer.q_temp,
+                                 v_first=None if v_first_cache is None else pool.get_value_buffer(v_first_cache),
+                                 v_mix=None if (v_first_cache is None or layer.v_mix is None) else layer.v_mix.data)
         if layer.block:
             kp, vp = pool.get_pooled_buffers(cache)
             _native.pool_blocks(kp, vp, kbuf, vbuf, forward_batch.req_to_token_pool.req_to_token, self.seq, layer.block)
 
-    def forward_window(self, q, layer: "PooledWindowAttention", forward_batch: "ForwardBatch", cache_id=None):
+    def forward_window(self, q, layer: "PooledWindowAttention", forward_batch: "ForwardBatch", cache_id=None, gate=None):
         pool = forward_batch.token_to_kv_pool
         cache = layer.layer_id if cache_id is None else cache_id
         kbuf, vbuf = pool.get_kv_buffer(cache)
@@ -629,7 +651,9 @@ class SequenceBackend(AttentionBackend):
         return _native.window_attention(q, kbuf, vbuf, kp, vp, forward_batch.req_to_token_pool.req_to_token, self.seq,
                                         layer.tp_q_head_num, layer.tp_k_head_num, layer.dim, layer.vdim, layer.window,
                                         layer.block, layer.scaling,
-                                        sinks=None if layer.sinks is None else layer.sinks.data)
+                                        sinks=None if layer.sinks is None else layer.sinks.data, softcap=layer.softcap,
+                                        sigmoid_weights=layer.sigmoid_weights,
+                                        head_bias=None if layer.head_bias is None else layer.head_bias.data, gate=gate)
 
     def forward_decode(self, q, k, v, layer, forward_batch, save_kv_cache: bool = True):
         raise NotImplementedError("this backend serves latent attention layers (forward_latent) and windowed ones (forward_window)")

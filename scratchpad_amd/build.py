@@ -32,7 +32,7 @@ PER_FILE_FLAGS = {"elementwise.hip": ["-ffp-contract=off"], "allreduce.hip": ["-
 # fp32 state and residual kernels: scalar fp32 instructions only (no packed-fp32 forms)
 _NO_PACKED_F32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unknown-warning-option"]
 for _f in ("scalar_norm.hip", "wkv.hip", "latent_attention.hip", "moe.hip", "stream_norm.hip", "window_attention.hip",
-           "ssm.hip", "mlstm.hip", "delta_rule.hip", "hgrn.hip"):
+           "ssm.hip", "mlstm.hip", "delta_rule.hip", "hgrn.hip", "gated_delta.hip"):
     PER_FILE_FLAGS[_f] = list(_NO_PACKED_F32)
 # Sources a model family needs beyond these: a model class names them (NATIVE_SOURCES) and build_native(only=...) makes
 # a library of just those, so the first start of a small model does not compile the attention kernels of another.

@@ -82,7 +82,7 @@ __global__ void moe_route_kernel(int32_t* ids, float* weights, const void* x, in
 // ---- softmax scores and choice on ready fp32 logits: one wave per token ---------------------------------------------
 // s = softmax(z) over all experts; the `top` largest s win (ties: the lower index); weights = s * scale
 __global__ void moe_softmax_topk_kernel(int32_t* ids, float* weights, const float* logits, int64_t T, int E, int top,
-                                        float scale) {
+                                        float scale, int renorm) {
   extern __shared__ float smem[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int64_t t = (int64_t)blockIdx.x * (blockDim.x >> 6) + wave;
@@ -102,6 +102,7 @@ __global__ void moe_softmax_topk_kernel(int32_t* ids, float* weights, const floa
     choice[e] = sv;
   }
   __builtin_amdgcn_wave_barrier();
+  float chosen = 0.f;                                  // lane 0: the sum of the chosen scores
   for (int k = 0; k < top; ++k) {
     float best = -INFINITY;
     int at = 0x7fffffff;
@@ -119,10 +120,14 @@ __global__ void moe_softmax_topk_kernel(int32_t* ids, float* weights, const floa
     if (lane == 0) {
       ids[t * top + k] = at;
       weights[t * top + k] = score[at] * scale;
+      chosen += score[at];
       choice[at] = -INFINITY;
     }
     __builtin_amdgcn_wave_barrier();
   }
+  // the softmax over the chosen logits only = the chosen scores divided by their sum
+  if (renorm && lane == 0)
+    for (int k = 0; k < top; ++k) weights[t * top + k] /= chosen;
 }
 
 // ---- pairs ordered by expert: offsets[E + 1], order[pos] = pair, place[pair] = pos.  One workgroup. ---------------
@@ -359,14 +364,15 @@ extern "C" int sp_moe_route(int32_t* ids, float* weights, const void* x, int64_t
 }
 
 extern "C" int sp_moe_softmax_topk(int32_t* ids, float* weights, const float* logits, int64_t num_tokens, int experts, int top,
-                                   float scale, void* stream) {
+                                   float scale, int renorm, void* stream) {
   SP_CHECK_ARG(num_tokens >= 0 && experts > 0 && top > 0 && top <= experts);
   if (num_tokens == 0) return SP_OK;
   SP_CHECK_ARG(ids && weights && logits);
   const size_t lds = 4 * (size_t)(2 * experts) * sizeof(float);
   if (lds > 64 * 1024) return SP_ERR_UNSUPPORTED;
   moe_softmax_topk_kernel<<<dim3((unsigned)((num_tokens + 3) / 4)), 256, lds, (hipStream_t)stream>>>(ids, weights, logits,
-                                                                                                  num_tokens, experts, top, scale);
+                                                                                                  num_tokens, experts, top, scale,
+                                                                                                  renorm);
   SP_LAUNCH_CHECK();
   return SP_OK;
 }

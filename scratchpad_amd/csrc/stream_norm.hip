@@ -9,6 +9,9 @@
 // and of sequential-sublayer models that gate and norm a sublayer's RESULT before it joins the stream:
 //   gated normed sum      y = a  or  (N(a) wa + N(b) wb) / 2;   y *= sigmoid(gate + gate_bias);   x += N(y) w;
 //                         x += extra;   next = N(x) w_next      (N = division by the row's root mean square)
+// and of sequential pre-norm models whose norm works in groups:
+//   sum + group norm      x += a  or  x += (N(a) wa + N(b) wb) / 2  (or nothing);   next = GN(x) w_next, GN = every one of
+//                         `groups` equal consecutive parts of the row divided by its own root mean square
 // All arithmetic is fp32; h and hs are rounded once, to the projections' element type.
 #include "seq_batch.h"
 
@@ -287,6 +290,54 @@ gated_add_norm_vec_kernel(float* x, int64_t x_stride, const void* a, int64_t a_s
   }
 }
 
+// one workgroup per row: the row's new x waits in LDS; wave w then forms the norm of the groups w, w + waves, ...
+template <typename Tag>
+__global__ void __launch_bounds__(kBlock)
+add_group_norm_kernel(float* x, int64_t x_stride, const void* a, int64_t a_stride, const float* wa, const void* b,
+                      int64_t b_stride, const float* wb, void* out_next, int64_t next_stride, const float* next_weight,
+                      int width, int groups, float eps) {
+  typedef Elem<Tag> E;
+  extern __shared__ float rowbuf[];                  // [width] the row, then [groups] the inverse roots
+  __shared__ float red[kBlock / 64];
+  float* ginv = rowbuf + width;
+  const int64_t t = blockIdx.x;
+  float ia = 1.f, ib = 0.f;
+  if (b) {
+    float sa = 0.f, sb = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+      const float u = E::load(a, t * a_stride + i), v = E::load(b, t * b_stride + i);
+      sa += u * u;
+      sb += v * v;
+    }
+    sa = block_sum(sa, red);
+    sb = block_sum(sb, red);
+    ia = 1.f / sqrtf(sa / (float)width + eps);
+    ib = 1.f / sqrtf(sb / (float)width + eps);
+  }
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float v = x[t * x_stride + i];
+    if (a) {
+      float y = E::load(a, t * a_stride + i);
+      if (b) y = 0.5f * (y * ia * wa[i] + E::load(b, t * b_stride + i) * ib * wb[i]);
+      v += y;
+      x[t * x_stride + i] = v;
+    }
+    rowbuf[i] = v;
+  }
+  if (!out_next) return;
+  __syncthreads();
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, per = width / groups;
+  for (int g = wave; g < groups; g += (int)(blockDim.x >> 6)) {
+    float ss = 0.f;
+    for (int i = lane; i < per; i += 64) ss += rowbuf[g * per + i] * rowbuf[g * per + i];
+    ss = wave_sum(ss);
+    if (lane == 0) ginv[g] = 1.f / sqrtf(ss / (float)per + eps);
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < width; i += blockDim.x)
+    E::store(out_next, t * next_stride + i, rowbuf[i] * ginv[i / per] * next_weight[i]);
+}
+
 }  // namespace
 }  // namespace sp
 
@@ -383,6 +434,24 @@ extern "C" int sp_gated_add_norm(float* x, int64_t x_stride, const void* a, int6
                                                           (hipStream_t)stream>>>(
                                x, x_stride, a, a_stride, wa, b, b_stride, wb, gate, gate_stride, gate_bias, weight, extra,
                                extra_stride, out_next, next_stride, next_weight, width, eps)));
+  SP_LAUNCH_CHECK();
+  return SP_OK;
+}
+
+extern "C" int sp_add_group_norm(float* x, int64_t x_stride, const void* a, int64_t a_stride, const float* wa, const void* b,
+                                 int64_t b_stride, const float* wb, void* out_next, int64_t next_stride,
+                                 const float* next_weight, int64_t num_tokens, int width, int groups, float eps, int dtype,
+                                 void* stream) {
+  SP_CHECK_ARG(num_tokens >= 0 && width > 0 && width <= 15360 && groups > 0 && groups <= 64 && width % groups == 0);
+  if (num_tokens == 0) return SP_OK;
+  SP_CHECK_ARG(x && x_stride >= width && (a || out_next));
+  SP_CHECK_ARG(!a || a_stride >= width);
+  SP_CHECK_ARG(!b || (a && wa && wb && b_stride >= width));
+  SP_CHECK_ARG(!out_next || (next_weight && next_stride >= width));
+  SP_DISPATCH_DTYPE(dtype, (add_group_norm_kernel<Tag><<<dim3((unsigned)num_tokens), kBlock,
+                                                          (size_t)(width + groups) * sizeof(float), (hipStream_t)stream>>>(
+                               x, x_stride, a, a_stride, wa, b, b_stride, wb, out_next, next_stride, next_weight, width,
+                               groups, eps)));
   SP_LAUNCH_CHECK();
   return SP_OK;
 }

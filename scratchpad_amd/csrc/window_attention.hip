@@ -15,6 +15,12 @@
 // and v before the rotation; the per-head norm of the values can be switched off.  Scores, softmax and the weighted sum are
 // fp32.  With `sinks` (one fp32 number per query head) the softmax's denominator holds one more term exp(sink): a key that
 // is seen by every query, is not scaled and has no value.
+//
+// Further forms of the same layer (each a parameter): q and k divided per head by their root mean square after the
+// rotation; q times a number per head and times 1 + coef ln(floor((position + 1) / every) + 1); values blended with the
+// values an earlier layer cached for the same token, v <- (1 - lambda) v + lambda v_first; scores capped as
+// cap tanh(score / cap); and, instead of the softmax, every visible key weighted by sigmoid(score + bias[head]) without
+// normalisation.  The result can be multiplied element by element with sigmoid(gate) on its way out.
 #include "seq_batch.h"
 
 namespace sp {
@@ -83,6 +89,110 @@ qkv_rotary_store_kernel(void* q, int64_t q_stride, const void* k, int64_t k_stri
   }
 }
 
+// The same store with a wave per head: q and k can be divided by their root mean square over the head AFTER the rotation
+// (qk_norm), q scaled per head and by position, v blended with the row another layer's pool holds for the same slot.
+// A lane holds the coordinates lane, lane + 64, ... of its head (dim, vdim <= 64 * kStorePerLane).
+constexpr int kStorePerLane = 4;
+template <typename Tag>
+__device__ __forceinline__ void rotated_head(float* val, const void* src, int64_t at, const float* bias, int col0, int D,
+                                             int dims, int adjacent, float pos, const float* freq, float mag, int lane) {
+  typedef Elem<Tag> E;
+  const int half = dims / 2;
+#pragma unroll
+  for (int u = 0; u < kStorePerLane; ++u) {
+    const int i = lane + 64 * u;
+    float out = 0.f;
+    if (i < D) {
+      const float x = E::load(src, at + i) + (bias ? bias[col0 + i] : 0.f);
+      out = x;
+      if (i < dims) {
+        int pi, fi;
+        bool first;
+        if (adjacent) {
+          first = (i & 1) == 0;
+          pi = first ? i + 1 : i - 1;
+          fi = i >> 1;
+        } else {
+          first = i < half;
+          pi = first ? i + half : i - half;
+          fi = first ? i : i - half;
+        }
+        const float y = E::load(src, at + pi) + (bias ? bias[col0 + pi] : 0.f);
+        const float ang = pos * freq[fi];
+        const float c = cosf(ang) * mag, sn = sinf(ang) * mag;
+        out = first ? x * c - y * sn : x * c + y * sn;
+      }
+    }
+    val[u] = out;
+  }
+}
+
+template <typename Tag>
+__global__ void __launch_bounds__(kBlock)
+qkv_norm_store_kernel(void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
+                      void* kpool, int64_t kp_stride, void* vpool, int64_t vp_stride, const int64_t* positions,
+                      const int64_t* loc, const float* freq, float mag, const float* qb, const float* kb, const float* vb,
+                      int H, int G, int D, int Dv, int dims, int adjacent, int norm_v, float eps, int qk_norm,
+                      const float* q_head_scale, float q_temp_coef, int q_temp_every, const void* v_first,
+                      int64_t vf_stride, const float* v_mix) {
+  typedef Elem<Tag> E;
+  const int64_t t = blockIdx.x;
+  const int64_t ipos = positions[t];
+  const float pos = (float)ipos;
+  const int64_t slot = loc[t];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, waves = blockDim.x >> 6;
+  float qmul = 1.f;
+  if (q_temp_every > 0) qmul = 1.f + q_temp_coef * logf((float)((ipos + 1) / q_temp_every) + 1.f);
+  for (int job = wave; job < H + 2 * G; job += waves) {
+    float val[kStorePerLane];
+    if (job < H + G) {
+      const bool isq = job < H;
+      const int h = isq ? job : job - H;
+      const void* src = isq ? q : k;
+      const int64_t at = t * (isq ? q_stride : k_stride) + (int64_t)h * D;
+      rotated_head<Tag>(val, src, at, isq ? qb : kb, h * D, D, dims, adjacent, pos, freq, mag, lane);
+      float mul = 1.f;
+      if (qk_norm) {
+        float ss = 0.f;
+#pragma unroll
+        for (int u = 0; u < kStorePerLane; ++u) ss += val[u] * val[u];       // (coordinates past D are zeros)
+        ss = wave_sum(ss);
+        mul = 1.f / sqrtf(ss / (float)D + eps);
+      }
+      if (isq) mul *= qmul * (q_head_scale ? q_head_scale[h] : 1.f);
+      void* dst = isq ? q : kpool;
+      const int64_t to = isq ? at : slot * kp_stride + (int64_t)h * D;
+#pragma unroll
+      for (int u = 0; u < kStorePerLane; ++u) {
+        const int i = lane + 64 * u;
+        if (i < D) E::store(dst, to + i, val[u] * mul);
+      }
+    } else {
+      const int g = job - H - G;
+      const int64_t at = t * v_stride + (int64_t)g * Dv, to = slot * vp_stride + (int64_t)g * Dv;
+      float ss = 0.f;
+#pragma unroll
+      for (int u = 0; u < kStorePerLane; ++u) {
+        const int i = lane + 64 * u;
+        val[u] = i < Dv ? E::load(v, at + i) + (vb ? vb[g * Dv + i] : 0.f) : 0.f;
+        ss += val[u] * val[u];
+      }
+      float mul = 1.f;
+      if (norm_v) mul = 1.f / sqrtf(wave_sum(ss) / (float)Dv + eps);
+      const float lam = v_first ? v_mix[0] : 0.f;
+#pragma unroll
+      for (int u = 0; u < kStorePerLane; ++u) {
+        const int i = lane + 64 * u;
+        if (i < Dv) {
+          float x = val[u] * mul;
+          if (v_first) x = (1.f - lam) * x + lam * E::load(v_first, slot * vf_stride + (int64_t)g * Dv + i);
+          E::store(vpool, to + i, x);
+        }
+      }
+    }
+  }
+}
+
 // a token that completes a block (position + 1 divisible by P) writes the block's mean key and value at its own slot
 template <typename Tag>
 __global__ void __launch_bounds__(kBlock)
@@ -134,12 +244,13 @@ __device__ __forceinline__ float dot_row(const float* sq, const void* base, int6
 // wave w takes tiles w, w + NW, ...: lane = key for the scores, lane = value channel for the
 // weighted sum (4 keys' rows in flight at a time); the waves' partial (maximum, sum, weighted values) meet in LDS.
 // The order of every sum depends on the query's position only, never on the batch or on how the prompt was cut.
-template <typename Tag, bool VEC>
+template <typename Tag, bool VEC, bool SIG>
 __global__ void __launch_bounds__(1024)
 window_attention_kernel(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kpool, const void* vpool,
                         const void* kpooled, const void* vpooled, int64_t kp_stride, int64_t vp_stride,
                         const int32_t* req_to_token, int64_t table_stride, SeqBatch s, int H, int G, int D, int Dv,
-                        int64_t size, int P, float scale, const float* sinks) {
+                        int64_t size, int P, float scale, const float* sinks, float softcap, const float* head_bias,
+                        const void* gate, int64_t gate_stride) {
   typedef Elem<Tag> E;
   extern __shared__ float smem[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, NW = blockDim.x >> 6;
@@ -161,6 +272,7 @@ window_attention_kernel(void* out, int64_t out_stride, const void* q, int64_t q_
   for (int i = threadIdx.x; i < D; i += blockDim.x) sq[i] = E::load(q, t * q_stride + (int64_t)h * D + i) * scale;
   __syncthreads();
   float m = -INFINITY, l = 0.f;
+  const float hbias = (SIG && head_bias) ? head_bias[h] : 0.f;
   float acc[kMaxPerLane];
 #pragma unroll
   for (int i = 0; i < kMaxPerLane; ++i) acc[i] = 0.f;
@@ -173,19 +285,25 @@ window_attention_kernel(void* out, int64_t out_stride, const void* q, int64_t q_
       const bool blk = kk < nb;
       const int64_t row = blk ? table[kk * P + P - 1] : table[w0 + (kk - nb)];
       sc = dot_row<Tag, VEC>(sq, blk ? kpooled : kpool, row * kp_stride + (int64_t)g * D, D);
+      if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);
     }
-    float tm = sc;
+    if constexpr (SIG) {                                // every visible key on its own: no maximum, no denominator
+      sw[lane] = lane < n ? 1.f / (1.f + expf(-(sc + hbias))) : 0.f;
+      __builtin_amdgcn_wave_barrier();
+    } else {
+      float tm = sc;
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) tm = fmaxf(tm, __shfl_xor(tm, off, 64));
-    const float m_new = fmaxf(m, tm);
-    const float corr = expf(m - m_new);                 // first tile: exp(-inf) = 0
-    const float p = lane < n ? expf(sc - m_new) : 0.f;
-    l = l * corr + wave_sum(p);
-    m = m_new;
-    sw[lane] = p;
-    __builtin_amdgcn_wave_barrier();
+      for (int off = 32; off > 0; off >>= 1) tm = fmaxf(tm, __shfl_xor(tm, off, 64));
+      const float m_new = fmaxf(m, tm);
+      const float corr = expf(m - m_new);                 // first tile: exp(-inf) = 0
+      const float p = lane < n ? expf(sc - m_new) : 0.f;
+      l = l * corr + wave_sum(p);
+      m = m_new;
+      sw[lane] = p;
+      __builtin_amdgcn_wave_barrier();
 #pragma unroll
-    for (int i = 0; i < kMaxPerLane; ++i) acc[i] *= corr;
+      for (int i = 0; i < kMaxPerLane; ++i) acc[i] *= corr;
+    }
     int j = 0;
     for (; j + 4 <= n; j += 4) {
       int64_t at[4];
@@ -233,6 +351,15 @@ window_attention_kernel(void* out, int64_t out_stride, const void* q, int64_t q_
     sml[NW + wave] = l;
   }
   __syncthreads();
+  if constexpr (SIG) {
+    for (int c = threadIdx.x; c < Dv; c += blockDim.x) {
+      float num = 0.f;
+      for (int w = 0; w < NW; ++w) num += sacc[w * Dv + c];
+      if (gate) num /= 1.f + expf(-E::load(gate, t * gate_stride + (int64_t)h * Dv + c));
+      E::store(out, t * out_stride + (int64_t)h * Dv + c, num);
+    }
+    return;
+  }
   float M = sml[0];                                                         // wave 0 always holds a key: M is finite
   for (int w = 1; w < NW; ++w) M = fmaxf(M, sml[w]);
   float den = 0.f;
@@ -245,7 +372,9 @@ window_attention_kernel(void* out, int64_t out_stride, const void* q, int64_t q_
   for (int c = threadIdx.x; c < Dv; c += blockDim.x) {
     float num = 0.f;
     for (int w = 0; w < NW; ++w) num += sacc[w * Dv + c] * expf(sml[w] - M);
-    E::store(out, t * out_stride + (int64_t)h * Dv + c, num * inv);
+    num *= inv;
+    if (gate) num /= 1.f + expf(-E::load(gate, t * gate_stride + (int64_t)h * Dv + c));
+    E::store(out, t * out_stride + (int64_t)h * Dv + c, num);
   }
 }
 
@@ -277,12 +406,13 @@ __device__ __forceinline__ f32x4_w mfma_w<f16_tag>(const u32x4& a, const u32x4& 
 
 constexpr int kVtRow = 72;      // 64 keys + 8 of padding per value channel (16-bit elements)
 
-template <typename Tag, int DS, int DT>      // DS = dim / 32, DT = vdim / 16
+template <typename Tag, int DS, int DT, bool SIG>      // DS = dim / 32, DT = vdim / 16
 __global__ void __launch_bounds__(256)
 window_attention_mfma_kernel(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kpool,
                              const void* vpool, const void* kpooled, const void* vpooled, int64_t kp_stride, int64_t vp_stride,
                              const int32_t* req_to_token, int64_t table_stride, SeqBatch s, int H, int G, int64_t size, int P,
-                             float scale, const float* sinks) {
+                             float scale, const float* sinks, float softcap, const float* head_bias, const void* gate,
+                             int64_t gate_stride) {
   constexpr int D = 32 * DS, Dv = 16 * DT;
   __shared__ uint16_t vt[Dv][kVtRow];
   __shared__ int32_t sslot[64];
@@ -313,6 +443,7 @@ window_attention_mfma_kernel(void* out, int64_t out_stride, const void* q, int64
   for (int h0 = 0; h0 < R; h0 += 4) {
     const int hq = g * R + h0 + wave;
     const bool work = h0 + wave < R;
+    const float hbias = (SIG && head_bias && work) ? head_bias[hq] : 0.f;
     u32x4 qf[DS];
 #pragma unroll
     for (int st = 0; st < DS; ++st)
@@ -374,29 +505,39 @@ window_attention_mfma_kernel(void* out, int64_t out_stride, const void* q, int64
                 vis = j >= w0_q && j <= pos_q;
               }
             }
-            const float v = vis ? sacc[sb][r] * scale : -INFINITY;
+            float v = vis ? sacc[sb][r] * scale : -INFINITY;
+            if (vis && softcap > 0.f) v = softcap * tanhf(v / softcap);
             sacc[sb][r] = v;
             mx = fmaxf(mx, v);
           }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m, mx);
-        const float m_safe = m_new == -INFINITY ? 0.f : m_new;      // nothing seen yet: every weight is exp(-inf) = 0
-        const float corr = expf(m - m_safe);
-        float psum = 0.f;
+        float corr = 1.f;
         float pf[2][8];
+        if constexpr (SIG) {                              // sigmoid(score + bias) per visible key, nothing to rescale
 #pragma unroll
-        for (int sb = 0; sb < 4; ++sb)
+          for (int sb = 0; sb < 4; ++sb)
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const float p = expf(sacc[sb][r] - m_safe);
-            psum += p;
-            pf[sb >> 1][4 * (sb & 1) + r] = p;
-          }
-        psum += __shfl_xor(psum, 16, 64);
-        psum += __shfl_xor(psum, 32, 64);
-        l = l * corr + psum;
-        m = m_new;
+            for (int r = 0; r < 4; ++r)
+              pf[sb >> 1][4 * (sb & 1) + r] = sacc[sb][r] == -INFINITY ? 0.f : 1.f / (1.f + expf(-(sacc[sb][r] + hbias)));
+        } else {
+          mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+          mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+          const float m_new = fmaxf(m, mx);
+          const float m_safe = m_new == -INFINITY ? 0.f : m_new;      // nothing seen yet: every weight is exp(-inf) = 0
+          corr = expf(m - m_safe);
+          float psum = 0.f;
+#pragma unroll
+          for (int sb = 0; sb < 4; ++sb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const float p = expf(sacc[sb][r] - m_safe);
+              psum += p;
+              pf[sb >> 1][4 * (sb & 1) + r] = p;
+            }
+          psum += __shfl_xor(psum, 16, 64);
+          psum += __shfl_xor(psum, 32, 64);
+          l = l * corr + psum;
+          m = m_new;
+        }
 #pragma unroll
         for (int hh = 0; hh < 2; ++hh) {
           // the weights enter the product as a 16-bit value plus a 16-bit remainder: they are never rounded to 8 bits of
@@ -409,7 +550,7 @@ window_attention_mfma_kernel(void* out, int64_t out_stride, const void* q, int64
           const u32x4 pr = pack16<Tag>(rest);
 #pragma unroll
           for (int dt = 0; dt < DT; ++dt) {
-            if (hh == 0) {
+            if (!SIG && hh == 0) {
 #pragma unroll
               for (int r = 0; r < 4; ++r) oacc[dt][r] *= corr;
             }
@@ -423,14 +564,24 @@ window_attention_mfma_kernel(void* out, int64_t out_stride, const void* q, int64
       }
     }
     if (work && qvalid) {
-      float inv = 1.f / l;
-      if (sinks) {                                     // (a valid query has seen itself: m is finite)
-        const float sk = sinks[hq], m2 = fmaxf(m, sk), keep = expf(m - m2);
-        inv = keep / (l * keep + expf(sk - m2));
+      float inv = 1.f;
+      if constexpr (!SIG) {
+        inv = 1.f / l;
+        if (sinks) {                                   // (a valid query has seen itself: m is finite)
+          const float sk = sinks[hq], m2 = fmaxf(m, sk), keep = expf(m - m2);
+          inv = keep / (l * keep + expf(sk - m2));
+        }
       }
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
         float f[8] = {oacc[dt][0] * inv, oacc[dt][1] * inv, oacc[dt][2] * inv, oacc[dt][3] * inv, 0.f, 0.f, 0.f, 0.f};
+        if (gate) {
+          float gf[8];
+          const u32x2 g2 = *(const u32x2*)((const char*)gate + ((t0 + r16) * gate_stride + (int64_t)hq * Dv + 16 * dt + 4 * qd) * 2);
+          unpack16<Tag>(u32x4{g2[0], g2[1], 0u, 0u}, gf);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) f[e] /= 1.f + expf(-gf[e]);
+        }
         const u32x4 pk = pack16<Tag>(f);
         *(u32x2*)((char*)out + ((t0 + r16) * out_stride + (int64_t)hq * Dv + 16 * dt + 4 * qd) * 2) = u32x2{pk[0], pk[1]};
       }
@@ -448,13 +599,25 @@ extern "C" int sp_qkv_rotary_store(void* q, int64_t q_stride, const void* k, int
                                    const int64_t* positions, const int64_t* loc, const float* freq, float mag,
                                    const float* q_bias, const float* k_bias, const float* v_bias, int64_t num_tokens,
                                    int heads, int kv_heads, int dim, int vdim, int rot_dims, int adjacent, int norm_values,
-                                   float eps, int dtype, void* stream) {
+                                   float eps, int qk_norm, const float* q_head_scale, float q_temp_coef, int q_temp_every,
+                                   const void* v_first, int64_t vf_stride, const float* v_mix, int dtype, void* stream) {
   SP_CHECK_ARG(num_tokens >= 0 && heads > 0 && kv_heads > 0 && dim > 0 && vdim > 0);
   SP_CHECK_ARG(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= dim);
   if (num_tokens == 0) return SP_OK;
   SP_CHECK_ARG(q && k && v && kpool && vpool && positions && loc && (freq || rot_dims == 0));
   SP_CHECK_ARG(q_stride >= (int64_t)heads * dim && k_stride >= (int64_t)kv_heads * dim && v_stride >= (int64_t)kv_heads * vdim);
   SP_CHECK_ARG(kp_stride >= (int64_t)kv_heads * dim && vp_stride >= (int64_t)kv_heads * vdim);
+  SP_CHECK_ARG(q_temp_every >= 0 && (!v_first || (v_mix && vf_stride >= (int64_t)kv_heads * vdim)));
+  if (qk_norm || q_head_scale || q_temp_every > 0 || v_first) {      // the wave-per-head form
+    if (dim > 64 * kStorePerLane || vdim > 64 * kStorePerLane) return SP_ERR_UNSUPPORTED;
+    SP_DISPATCH_DTYPE(dtype, (qkv_norm_store_kernel<Tag><<<dim3((unsigned)num_tokens), kBlock, 0, (hipStream_t)stream>>>(
+                                 q, q_stride, k, k_stride, v, v_stride, kpool, kp_stride, vpool, vp_stride, positions, loc,
+                                 freq, mag, q_bias, k_bias, v_bias, heads, kv_heads, dim, vdim, rot_dims, adjacent,
+                                 norm_values, eps, qk_norm, q_head_scale, q_temp_coef, q_temp_every, v_first, vf_stride,
+                                 v_mix)));
+    SP_LAUNCH_CHECK();
+    return SP_OK;
+  }
   SP_DISPATCH_DTYPE(dtype, (qkv_rotary_store_kernel<Tag><<<dim3((unsigned)num_tokens), kBlock, 0, (hipStream_t)stream>>>(
                                q, q_stride, k, k_stride, v, v_stride, kpool, kp_stride, vpool, vp_stride, positions, loc,
                                freq, mag, q_bias, k_bias, v_bias, heads, kv_heads, dim, vdim, rot_dims, adjacent, norm_values,
@@ -484,7 +647,9 @@ extern "C" int sp_window_attention(void* out, int64_t out_stride, const void* q,
                                    const void* vpool, const void* kpooled, const void* vpooled, int64_t kp_stride,
                                    int64_t vp_stride, const int32_t* req_to_token, int64_t table_stride,
                                    int64_t num_tokens, int heads, int kv_heads, int dim, int vdim, int64_t window, int block,
-                                   float scale, const float* sinks, int matrix, SP_SEQ_PARAMS, int dtype, void* stream) {
+                                   float scale, const float* sinks, float softcap, int sigmoid_weights,
+                                   const float* head_bias, const void* gate, int64_t gate_stride, int matrix, SP_SEQ_PARAMS,
+                                   int dtype, void* stream) {
   SP_CHECK_ARG(num_tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0);
   if (num_tokens == 0) return SP_OK;
   SP_CHECK_ARG(out && q && kpool && vpool && req_to_token && req_pool_indices && seq_lens);
@@ -493,6 +658,8 @@ extern "C" int sp_window_attention(void* out, int64_t out_stride, const void* q,
   SP_CHECK_ARG(extend_seq_lens || num_tokens == batch_size);
   SP_CHECK_ARG(q_stride >= (int64_t)heads * dim && out_stride >= (int64_t)heads * vdim);
   SP_CHECK_ARG(kp_stride >= (int64_t)kv_heads * dim && vp_stride >= (int64_t)kv_heads * vdim);
+  SP_CHECK_ARG(!gate || gate_stride >= (int64_t)heads * vdim);
+  SP_CHECK_ARG(!sigmoid_weights || !sinks);
   if (vdim > 64 * kMaxPerLane) return SP_ERR_UNSUPPORTED;
   const int nw = extend_seq_lens ? 4 : 16;       // waves per (token, head): see the kernel
   const size_t lds = ((size_t)dim + 64 * nw + (size_t)nw * vdim + 2 * nw) * sizeof(float);
@@ -502,12 +669,18 @@ extern "C" int sp_window_attention(void* out, int64_t out_stride, const void* q,
   const bool al16 = (((uintptr_t)q | (uintptr_t)kpool | (uintptr_t)vpool | (uintptr_t)kpooled | (uintptr_t)vpooled) & 15) == 0 &&
                     ((uintptr_t)out & 7) == 0;
   if (matrix && extend_seq_lens && num_tokens > batch_size && (dtype == SP_BF16 || dtype == SP_F16) && (dim == 64 || dim == 128) &&
-      (vdim == 64 || vdim == 128) && al16 && q_stride % 8 == 0 && kp_stride % 8 == 0 && vp_stride % 8 == 0 && out_stride % 4 == 0) {
+      (vdim == 64 || vdim == 128) && al16 && q_stride % 8 == 0 && kp_stride % 8 == 0 && vp_stride % 8 == 0 && out_stride % 4 == 0 &&
+      (!gate || (((uintptr_t)gate & 7) == 0 && gate_stride % 4 == 0))) {
     const dim3 mgrid((unsigned)((num_tokens + 15) / 16 + batch_size), (unsigned)kv_heads);
-#define SP_WM(T, DS, DT)                                                                                                 \
-  window_attention_mfma_kernel<T, DS, DT><<<mgrid, 256, 0, (hipStream_t)stream>>>(                                         \
+#define SP_WM2(T, DS, DT, SG)                                                                                            \
+  window_attention_mfma_kernel<T, DS, DT, SG><<<mgrid, 256, 0, (hipStream_t)stream>>>(                                     \
       out, out_stride, q, q_stride, kpool, vpool, kpooled, vpooled, kp_stride, vp_stride, req_to_token, table_stride, s, heads, \
-      kv_heads, window, block, scale, sinks)
+      kv_heads, window, block, scale, sinks, softcap, head_bias, gate, gate_stride)
+#define SP_WM(T, DS, DT)                    \
+  do {                                      \
+    if (sigmoid_weights) SP_WM2(T, DS, DT, true); \
+    else SP_WM2(T, DS, DT, false);          \
+  } while (0)
 #define SP_WM_SHAPES(T)                                   \
   do {                                                    \
     if (dim == 64 && vdim == 64) SP_WM(T, 2, 4);          \
@@ -519,6 +692,7 @@ extern "C" int sp_window_attention(void* out, int64_t out_stride, const void* q,
     else SP_WM_SHAPES(f16_tag);
 #undef SP_WM_SHAPES
 #undef SP_WM
+#undef SP_WM2
     SP_LAUNCH_CHECK();
     return SP_OK;
   }
@@ -526,12 +700,15 @@ extern "C" int sp_window_attention(void* out, int64_t out_stride, const void* q,
   const int vecn = dtype == SP_F32 ? 4 : 8;
   const bool vec = dim % vecn == 0 && kp_stride % vecn == 0 && ((uintptr_t)kpool & 15) == 0 &&
                    (!kpooled || ((uintptr_t)kpooled & 15) == 0);
-#define SP_WA(V)                                                                                                       \
-  SP_DISPATCH_DTYPE(dtype, (window_attention_kernel<Tag, V><<<grid, 64 * nw, lds, (hipStream_t)stream>>>(               \
+#define SP_WA(V, SG)                                                                                                   \
+  SP_DISPATCH_DTYPE(dtype, (window_attention_kernel<Tag, V, SG><<<grid, 64 * nw, lds, (hipStream_t)stream>>>(           \
                                out, out_stride, q, q_stride, kpool, vpool, kpooled, vpooled, kp_stride, vp_stride,      \
-                               req_to_token, table_stride, s, heads, kv_heads, dim, vdim, window, block, scale, sinks)))
-  if (vec) SP_WA(true);
-  else SP_WA(false);
+                               req_to_token, table_stride, s, heads, kv_heads, dim, vdim, window, block, scale, sinks,  \
+                               softcap, head_bias, gate, gate_stride)))
+  if (vec && sigmoid_weights) SP_WA(true, true);
+  else if (vec) SP_WA(true, false);
+  else if (sigmoid_weights) SP_WA(false, true);
+  else SP_WA(false, false);
 #undef SP_WA
   SP_LAUNCH_CHECK();
   return SP_OK;

@@ -391,6 +391,32 @@ class GatedAddNorm(nn.Module):
                                       extra=extra, next_weight=next_weight)
 
 
+class GroupRMSNorm(nn.Module):
+    """Weighted RMS norm of an fp32 residual stream taken in ``groups`` equal consecutive parts of the row, each divided by
+    its own root mean square; fused with the sum that precedes it in a pre-norm layer: ``forward(x, dtype, y)`` adds a
+    sublayer's result y to the stream in place first (two branches (a, b) with ``branch_weights`` (wa, wb): each normed
+    over the whole row with its weight, then averaged) and returns GN(x) * weight in the projections' dtype."""
+
+    def __init__(self, width: int, groups: int = 1, eps: float = 1e-6) -> None:
+        super().__init__()
+        if width % groups:
+            raise ValueError("the width must divide into the norm's groups")
+        self.weight = nn.Parameter(torch.ones(width, dtype=torch.float32), requires_grad=False)
+        self.groups, self.variance_epsilon = groups, eps
+
+    def forward(self, x: torch.Tensor, dtype: torch.dtype, y=None, branch_weights=None) -> torch.Tensor:
+        return add_join(x, y, branch_weights, self.groups, self.variance_epsilon, dtype, self.weight.data)
+
+
+def add_join(x: torch.Tensor, y, branch_weights, groups: int, eps: float, dtype: torch.dtype,
+             next_weight: Optional[torch.Tensor] = None):
+    """x += y in place (y one tensor, or two branches each normed over the row with its weight and averaged), then,
+    with ``next_weight``, the group norm of the new x times that weight"""
+    a, b = y if isinstance(y, (tuple, list)) else (y, None)
+    wa, wb = branch_weights if b is not None else (None, None)
+    return _native.add_group_norm(x, a, groups, eps, dtype, b=b, wa=wa, wb=wb, next_weight=next_weight)
+
+
 class ReluSquareFF(nn.Module):
     """Feed-forward W_down relu(W_up h)^2.  ``extra_rows`` further rows of the up projection are not activated: their
     outputs come back beside the result (a layer's gate on this sublayer reads the same h, so it rides in this product)."""

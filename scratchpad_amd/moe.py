@@ -58,15 +58,18 @@ class SparseMoE(nn.Module):
 
 class SoftmaxRouter(nn.Module):
     """ids, weights = the `top` experts with the largest softmax(W x) over ALL experts (fp32 logits); the weights are
-    those scores times `scale`, not renormalised over the chosen ones."""
+    those scores times `scale`, not renormalised over the chosen ones.  ``bias``: the logits are W x + b.  ``renorm``:
+    the weights are the softmax over the CHOSEN logits only (they sum to `scale`)."""
 
-    def __init__(self, width: int, experts: int, top: int, scale: float = 1.0):
+    def __init__(self, width: int, experts: int, top: int, scale: float = 1.0, bias: bool = False, renorm: bool = False):
         super().__init__()
-        self.experts, self.top, self.scale = experts, top, scale
+        self.experts, self.top, self.scale, self.renorm = experts, top, scale, renorm
         self.weight = nn.Parameter(torch.zeros(experts, width, dtype=torch.float32), requires_grad=False)
+        self.bias = nn.Parameter(torch.zeros(experts, dtype=torch.float32), requires_grad=False) if bias else None
 
     def forward(self, x: torch.Tensor):
-        return _native.moe_route_softmax(x, self.weight.data, self.top, self.scale)
+        return _native.moe_route_softmax(x, self.weight.data, self.top, self.scale,
+                                         None if self.bias is None else self.bias.data, self.renorm)
 
 
 class SiluGluExperts(ClampedGluExperts):
@@ -87,6 +90,20 @@ class SoftmaxMoE(nn.Module):
         super().__init__()
         self.router = SoftmaxRouter(width, experts, top, scale)
         self.experts = SiluGluExperts(width, experts, ff, dtype=dtype)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        ids, weights = self.router(x)
+        return self.experts(x, ids, weights)
+
+
+class ChosenSoftmaxMoE(nn.Module):
+    """Experts chosen by the largest router logits W x + b and weighted by the softmax over the chosen logits only, each a
+    clamped gated unit (ClampedGluExperts); `forward` returns their weighted sum."""
+
+    def __init__(self, width: int, experts: int, top: int, ff: int, limit: float, dtype=None):
+        super().__init__()
+        self.router = SoftmaxRouter(width, experts, top, bias=True, renorm=True)
+        self.experts = ClampedGluExperts(width, experts, ff, limit, dtype=dtype)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         ids, weights = self.router(x)

@@ -1,7 +1,7 @@
 """Recurrent token mixers over per-request state in the RecurrentStatePool: WKVMixer (RWKV-style time mixing, csrc/wkv.hip),
 Mamba2Mixer (state-space duality form, csrc/ssm.hip), MLSTMMixer (matrix memory with exponential gating, csrc/mlstm.hip),
-GeneralDeltaMixer (generalized delta rule, csrc/delta_rule.hip) and HGRN2Mixer (linear attention whose forget gate also
-writes, csrc/hgrn.hip).
+GeneralDeltaMixer (generalized delta rule, csrc/delta_rule.hip), HGRN2Mixer (linear attention whose forget gate also
+writes, csrc/hgrn.hip) and GatedDeltaMixer (delta rule with a decay per key channel, csrc/gated_delta.hip).
 
 WKVMixer:
 
@@ -204,6 +204,58 @@ class HGRN2Mixer(nn.Module):
         S = states.state(self.layer_id if state_id is None else state_id, "S")
         o = _native.hgrn2_scan(a[:, :nk], a[:, nk:2 * nk], a[:, 2 * nk:self.in_rows], self.f_bias.data, self.lower.data,
                                self.norm.data, S, seq, self.heads, self.dim, self.vdim, self.eps)
+        return _native.linear(o, self.o)
+
+    def forward(self, h: torch.Tensor, forward_batch: ForwardBatch, state_id: Optional[int] = None) -> torch.Tensor:
+        return self.scan(_native.linear(h, self.in_proj), forward_batch, state_id)
+
+
+class GatedDeltaMixer(nn.Module):
+    """Delta rule with a decay per head and key channel.  q, k [kv_heads, dim] and v [heads, vdim] are projections of h that
+    pass a causal per-channel convolution of ``taps`` taps (no bias; its latest taps - 1 inputs are request state) and silu;
+    value head h reads query/key head h // (heads / kv_heads).  In fp32, per head:
+        qn = q / sqrt(|q|^2 + 1e-6) dim^(-1/2),   kn = k / sqrt(|k|^2 + 1e-6),   beta = sigmoid(W_b h)
+        w  = exp(-exp(A_log) softplus(W_a2 (W_a1 h) + dt_bias))                    [dim] per head
+        S <- diag(w) S;   u = beta (v - S^T kn);   S <- S + kn u^T;   o = S^T qn   (S [dim, vdim])
+    out = W_o (o / rms_head(o) * norm * sigmoid(W_g2 (W_g1 h))), norm [vdim] shared by the heads.  The rows
+    [q | k | v | b | a1 | g1] of the input projection may be part of a larger product of the caller (``scan`` takes the
+    views); ``forward`` runs the mixer's own.  The second projections of decay and gate are fp32."""
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int, vdim: int, taps: int, decay_rank: int, gate_rank: int,
+                 eps: float, layer_id: Optional[int] = None, own_input: bool = True, dtype=None):
+        super().__init__()
+        if heads % kv_heads:
+            raise ValueError("value heads must be a multiple of query/key heads")
+        self.heads, self.kv_heads, self.dim, self.vdim, self.taps, self.eps = heads, kv_heads, dim, vdim, taps, eps
+        self.decay_rank, self.gate_rank, self.layer_id = decay_rank, gate_rank, layer_id
+        self.conv_rows = 2 * kv_heads * dim + heads * vdim
+        self.in_rows = self.conv_rows + heads + decay_rank + gate_rank
+        f32 = dict(dtype=torch.float32)
+        self.in_proj = nn.Parameter(torch.empty(self.in_rows, width, dtype=dtype), requires_grad=False) if own_input else None
+        self.conv = nn.Parameter(torch.zeros(self.conv_rows, taps, **f32), requires_grad=False)
+        self.a2t = nn.Parameter(torch.zeros(decay_rank, heads * dim, **f32), requires_grad=False)      # W_a2 transposed
+        self.dt_bias = nn.Parameter(torch.zeros(heads * dim, **f32), requires_grad=False)
+        self.A_log = nn.Parameter(torch.zeros(heads, **f32), requires_grad=False)
+        self.g2t = nn.Parameter(torch.zeros(gate_rank, heads * vdim, **f32), requires_grad=False)      # W_g2 transposed
+        self.norm = nn.Parameter(torch.ones(vdim, **f32), requires_grad=False)
+        self.o = nn.Parameter(torch.empty(width, heads * vdim, dtype=dtype), requires_grad=False)
+
+    @staticmethod
+    def state_shapes(heads: int, kv_heads: int, dim: int, vdim: int, taps: int):
+        return {"S": (heads, dim, vdim), "conv": (max(taps - 1, 0), 2 * kv_heads * dim + heads * vdim)}
+
+    def scan(self, a: torch.Tensor, forward_batch: ForwardBatch, state_id: Optional[int] = None) -> torch.Tensor:
+        """a [T, >= in_rows]: the outputs of the rows [q | k | v | b | a1 | g1] -> the mixer's output [T, W]"""
+        seq, states = forward_batch.attn_backend.seq, forward_batch.state_pool
+        sid = self.layer_id if state_id is None else state_id
+        nk, H, c = self.kv_heads * self.dim, self.heads, self.conv_rows
+        qkv = _native.causal_conv_silu(a[:, :c], self.conv.data, None, states.state(sid, "conv"), seq)
+        decay = _native.lowrank_gate(a[:, c + H:c + H + self.decay_rank], self.a2t.data, self.dt_bias.data, "decay",
+                                     self.A_log.data)
+        gate = _native.lowrank_gate(a[:, c + H + self.decay_rank:self.in_rows], self.g2t.data, None, "sigmoid")
+        o = _native.gated_delta_scan(qkv[:, :nk], qkv[:, nk:2 * nk], qkv[:, 2 * nk:], a[:, c:c + H], decay, gate,
+                                     self.norm.data, states.state(sid, "S"), seq, H, self.kv_heads, self.dim, self.vdim,
+                                     self.eps)
         return _native.linear(o, self.o)
 
     def forward(self, h: torch.Tensor, forward_batch: ForwardBatch, state_id: Optional[int] = None) -> torch.Tensor:

@@ -40,6 +40,11 @@ def _toredra_config(raw: dict, context_len=None, tensor_shapes=None, **_kw):
     return ToredraConfig(raw, context_len=context_len or 8192, tensor_shapes=tensor_shapes)
 
 
+def _kikurax_config(raw: dict, context_len=None, tensor_shapes=None, **_kw):
+    from .kikurax import KikuraxConfig
+    return KikuraxConfig(raw, context_len=context_len or 8192, tensor_shapes=tensor_shapes)
+
+
 def _llama_class():
     from .llama import LlamaForCausalLM
     return LlamaForCausalLM
@@ -65,6 +70,11 @@ def _toredra_class():
     return ToredraForCausalLM
 
 
+def _kikurax_class():
+    from .kikurax import KikuraxForCausalLM
+    return KikuraxForCausalLM
+
+
 # architecture name -> (configuration from config.json's dict, model class); both lazy so that naming a model does not
 # import the others
 MODELS = {
@@ -72,6 +82,7 @@ MODELS = {
     "Tizalorn": (_tizalorn_config, _tizalorn_class),
     "Sominex": (_sominex_config, _sominex_class),
     "Toredra": (_toredra_config, _toredra_class),
+    "Kikurax": (_kikurax_config, _kikurax_class),
 }
 
 
