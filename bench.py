@@ -70,7 +70,7 @@ def parse_args():
     ap.add_argument("--sample", action="store_true",
                     help="serve mode: temperature 0.8 / top-p 0.9 / top-k 50 sampling instead of greedy")
     ap.add_argument("--rate", type=float, default=0.0, help="serve mode: Poisson arrival rate (req/s); 0 = all at t=0")
-    ap.add_argument("--mode", default="decode", choices=["decode", "prefill", "serve", "tp", "hybrid", "sominex", "toredra"],
+    ap.add_argument("--mode", default="decode", choices=["decode", "prefill", "serve", "tp", "hybrid", "sominex", "toredra", "kikurax"],
                     help="decode = the headline metric (+ the TTFT half); prefill = config 3 alone; "
                          "tp = config 4 (sharded model, RCCL); hybrid = the Tizalorn design (recurrent + latent-attention "
                          "+ expert layers) beside a Llama of equal width and depth, with a per-kernel roofline table "
@@ -78,7 +78,7 @@ def parse_args():
                          "pooled blocks, Mamba-2 and mLSTM layers, softmax-routed experts); toredra = the Toredra design "
                          "(generalized delta rule layers, attention with a sink beside a forget-write linear attention, gated "
                          "and normed sublayer results) beside Sominex and Llama layers of equal width and depth")
-    ap.add_argument("--sizes", default="l", help="hybrid / sominex / toredra mode: model widths to run, of s (1024), m (2048) and l (4096)")
+    ap.add_argument("--sizes", default="l", help="hybrid / sominex / toredra / kikurax mode: model widths to run, of s (1024), m (2048) and l (4096)")
     ap.add_argument("--no-kernel-table", action="store_true", help="hybrid mode: throughput only")
     ap.add_argument("--graph", action="store_true",
                     help="hybrid mode: replay captured decode steps (default: eager launches for both models; a model class "
@@ -893,7 +893,7 @@ def tp_main(args, rank, local_rank, world):
 
 def main():
     args = parse_args()
-    if args.mode in ("hybrid", "sominex", "toredra"):   # (a parent of one child process per model: nothing here touches the GPU)
+    if args.mode in ("hybrid", "sominex", "toredra", "kikurax"):   # (a parent of one child process per model: nothing here touches the GPU)
         if args.gpus != 1:
             raise SystemExit(f"--mode {args.mode} is a one-GPU comparison")
         from bench_hybrid import hybrid_main

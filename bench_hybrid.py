@@ -1,6 +1,7 @@
-"""bench.py --mode hybrid / --mode sominex / --mode toredra: prefill and decode throughput of the Tizalorn / the Sominex / the
-Toredra design at layer sizes of real models (random weights), beside a Llama of the same width and depth on the same engine
-path (the Toredra mode also runs Sominex, its nearest relative), and a per-kernel table: every HIP kernel
+"""bench.py --mode hybrid / --mode sominex / --mode toredra / --mode kikurax: prefill and decode throughput of the Tizalorn /
+the Sominex / the Toredra / the Kikurax design at layer sizes of real models (random weights), beside a Llama of the same
+width and depth on the same engine path (the Toredra mode also runs Sominex, the Kikurax mode Sominex and Toredra: their
+nearest relatives), and a per-kernel table: every HIP kernel
 (and library product) of both models timed inside an eager prefill batch and an eager decode step, with the time its
 algorithmic bytes and flops would take at the chip's peaks (fraction of roofline).
 
@@ -71,6 +72,27 @@ def toredra_config(width: int, layers: int, context_len: int):
     raw = {"architecture": "Toredra", "vocab": 128256, "width": width, "norm": {"eps": 1e-5}, "logit_scale": 0.5,
            "logit_softcap": 50.0, "layers": [{**pattern[i % 4], "mlp": dense} for i in range(layers)]}
     return ToredraConfig(raw, context_len=context_len, decay_rank=64)
+
+
+def kikurax_config(width: int, layers: int, context_len: int):
+    """layers in the order attention, parallel, mamba2, parallel, each with 32 experts of which 4: attention heads of 128 with
+    a quarter as many key/value heads and rotation on half of each head; sigmoid attention of the same shape beside a
+    channel-gated delta rule of width / 128 heads with 128 x 128 states over width / 256 query/key heads (rank-64 decay and
+    gate projections, 4 taps); Mamba-2 as in the Sominex configuration"""
+    from scratchpad_amd.kikurax import KikuraxConfig
+    heads = {"heads": width // 128, "kv_heads": max(1, width // 512), "dim": 128, "vdim": 128}
+    att = {"type": "attention",
+           "mixer": {**heads, "scale": 0.09, "softcap": 30.0, "v_mix": True,
+                     "rot": {"base": 500000.0, "dims": 64, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 4096}}}}
+    par = {"type": "parallel",
+           "mixer": {"left": {**heads, "scale": 0.09, "q_temp": {"coef": 0.5, "every": 256}},
+                     "right": {"heads": width // 128, "kv_heads": max(1, width // 256), "dim": 128, "vdim": 128, "conv": 4}}}
+    mam = {"type": "mamba2", "mixer": {"heads": 2 * width // 64, "vdim": 64, "state": 128, "groups": 8, "conv": 4, "norm_groups": 8}}
+    moe = {"kind": "moe", "expert": {"ff": width // 2, "limit": 7.0}, "router": {"experts": 32, "top": 4}}
+    pattern = [att, par, mam, par]
+    raw = {"architecture": "Kikurax", "vocab": 128256, "width": width, "norm": {"eps": 1e-5, "groups": 4},
+           "embedding": {"scale": float(width) ** 0.5}, "layers": [{**pattern[i % 4], "mlp": moe} for i in range(layers)]}
+    return KikuraxConfig(raw, context_len=context_len, low_rank=64)
 
 
 def llama_config(width: int, layers: int, context_len: int):
@@ -205,6 +227,14 @@ def instrument(clock: KernelClock, cfg):
         H, D, Hkv = q.shape[1], q.shape[2], kb.shape[1]
         return _nbytes(o, q) + clock.keys_read() * 2 * Hkv * D * kb.element_size(), 4 * H * D * clock.pairs(), MATRIX
 
+    def gdelta(a, k, out):       # one sweep per token: the update (2 flops per state element), the read-out (2), the next u^T S (2)
+        q, state, heads, D, Dv = a[0], a[7], a[9], a[11], a[12]
+        return _nbytes(*a[:6], out) + 2 * len(clock.step["extend"]) * heads * D * Dv * 4, 6 * q.shape[0] * heads * D * Dv, VECTOR32
+
+    def lowrank(a, k, out):
+        p, w = a[0], a[1]
+        return _nbytes(p, w, out), 2 * p.shape[0] * w.shape[0] * w.shape[1], VECTOR32
+
     costs = {"embed_bigram_norm": io, "add_scalar_norm": io, "scalar_norm": io, "polynorm": io, "gate_heads": io,
              "token_shift": io, "wkv_decay": io, "wkv_recurrence": wkv, "rotary_interleaved": io, "latent_kv_store": io,
              "latent_attention": latent, "moe_route": io, "moe_align": io, "moe_grouped_gemm": grouped, "moe_glu": io,
@@ -214,7 +244,7 @@ def instrument(clock: KernelClock, cfg):
              "window_attention": window, "small_linear_f32": small, "causal_conv_silu": io, "mamba2_scan": scan,
              "gated_group_norm": io, "mlstm_scan": mlstm, "moe_route_softmax": io,
              "gated_add_norm": io, "relu_square": io, "scale_softcap": io, "delta_gates": io, "delta_recurrence": delta,
-             "hgrn2_scan": hgrn}
+             "hgrn2_scan": hgrn, "add_group_norm": io, "lowrank_gate": lowrank, "gated_delta_scan": gdelta}
     for name, cost in costs.items():
         saved[name] = getattr(N, name)
         setattr(N, name, clock.record(name, saved[name], cost))
@@ -343,7 +373,8 @@ def hybrid_main(args, design: str = "tizalorn"):
     runs = []
     for w in widths:
         row = {"width": w, "layers": layers}
-        for model in ((design, "sominex", "llama") if design == "toredra" else (design, "llama")):
+        beside = {"toredra": ("sominex", "llama"), "kikurax": ("sominex", "toredra", "llama")}.get(design, ("llama",))
+        for model in (design, *beside):
             cmd = [sys.executable, "-u", os.path.abspath(__file__), "--child", model, "--width", str(w), "--layers", str(layers),
                    "--bs", str(args.bs), "--ctx", str(args.ctx), "--steps", str(args.steps), "--warmup", str(args.warmup),
                    "--max-prefill-tokens", str(args.max_prefill_tokens)]
@@ -375,7 +406,7 @@ def child_main():
     import sys
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
     ap = argparse.ArgumentParser()
-    ap.add_argument("--child", required=True, choices=["tizalorn", "sominex", "toredra", "llama"])
+    ap.add_argument("--child", required=True, choices=["tizalorn", "sominex", "toredra", "kikurax", "llama"])
     for name in ("width", "layers", "bs", "ctx", "steps", "warmup", "max-prefill-tokens"):
         ap.add_argument("--" + name, type=int, required=True)
     ap.add_argument("--no-graph", action="store_true")
@@ -385,7 +416,7 @@ def child_main():
         raise SystemExit(DISABLED)
     torch.cuda.set_device(0)
     ctx_len = a.ctx + 2 * (a.steps + a.warmup) + 16
-    cfg = {"sominex": sominex_config, "toredra": toredra_config, "llama": llama_config}[a.child](a.width, a.layers, ctx_len)
+    cfg = {"sominex": sominex_config, "toredra": toredra_config, "kikurax": kikurax_config, "llama": llama_config}[a.child](a.width, a.layers, ctx_len)
     out = run_model(cfg, a, not a.no_kernel_table)
     print("RESULT " + json.dumps(out), flush=True)
 

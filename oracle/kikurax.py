@@ -243,3 +243,92 @@ def forward(tokens: List[int], w: Dict[str, torch.Tensor], cfg: dict, layers_out
         if layers_out is not None:
             layers_out.append(x.clone())
     return group_norm(x, w["final.norm"], groups, eps) @ w["embed"].T
+
+
+# ----------------------------------------------------------------------------------------------- random weights
+def tensor_shapes(cfg: dict, rank_a: int = 6, rank_g: int = 10) -> Dict[str, tuple]:
+    """name -> shape of a checkpoint of the design; the ranks of the right mixer's low-rank projections are given by a
+    checkpoint's tensor shapes only"""
+    W, V = int(cfg["width"]), int(cfg["vocab"])
+    s = {"embed": (V, W), "final.norm": (W,)}
+    for i, spec in enumerate(cfg["layers"]):
+        p, m = f"l{i}", spec["mixer"]
+        s[f"{p}.norm1"] = (W,)
+        if spec["type"] == "attention":
+            H, G, D, Dv = (int(m[k]) for k in ("heads", "kv_heads", "dim", "vdim"))
+            for n, rows in (("q", H * D), ("k", G * D), ("v", G * Dv)):
+                s[f"{p}.mix.{n}"] = (rows, W)
+                s[f"{p}.mix.{n}.b"] = (rows,)
+            s[f"{p}.mix.temp"] = (H,)
+            if m.get("v_mix"):
+                s[f"{p}.mix.vmix"] = ()
+            s[f"{p}.mix.o"] = (W, H * Dv)
+        elif spec["type"] == "mamba2":
+            H, Dv, N, G, K = (int(m[k]) for k in ("heads", "vdim", "state", "groups", "conv"))
+            inner, ch = H * Dv, H * Dv + 2 * G * N
+            s[f"{p}.mix.in"] = (inner + ch + H, W)
+            s[f"{p}.mix.conv"], s[f"{p}.mix.conv.b"] = (ch, K), (ch,)
+            s[f"{p}.mix.dt_bias"] = s[f"{p}.mix.A_log"] = s[f"{p}.mix.D"] = (H,)
+            s[f"{p}.mix.norm"] = (inner,)
+            s[f"{p}.mix.o"] = (W, inner)
+        else:
+            a, b = m["left"], m["right"]
+            H, G, D, Dv = (int(a[k]) for k in ("heads", "kv_heads", "dim", "vdim"))
+            L, R = f"{p}.mix.left", f"{p}.mix.right"
+            s[f"{L}.q"], s[f"{L}.k"], s[f"{L}.v"], s[f"{L}.g"] = (H * D, W), (G * D, W), (G * Dv, W), (H * Dv, W)
+            s[f"{L}.pb"] = (H,)
+            s[f"{L}.o"] = (W, H * Dv)
+            H, G, D, Dv, K = (int(b[k]) for k in ("heads", "kv_heads", "dim", "vdim", "conv"))
+            for n, rows in (("q", G * D), ("k", G * D), ("v", H * Dv)):
+                s[f"{R}.{n}"] = (rows, W)
+                s[f"{R}.{n}.conv"] = (rows, K)
+            s[f"{R}.b"] = (H, W)
+            s[f"{R}.A_log"] = (H,)
+            s[f"{R}.norm"] = (Dv,)
+            s[f"{R}.a1"], s[f"{R}.a2"], s[f"{R}.dt_bias"] = (rank_a, W), (H * D, rank_a), (H * D,)
+            s[f"{R}.g1"], s[f"{R}.g2"] = (rank_g, W), (H * Dv, rank_g)
+            s[f"{R}.o"] = (W, H * Dv)
+            s[f"{L}.out"] = s[f"{R}.out"] = (W,)
+        mlp = spec.get("mlp")
+        if mlp is not None:
+            s[f"{p}.norm2"] = (W,)
+            ff, E = int(mlp["expert"]["ff"]), int(mlp["router"]["experts"])
+            for e in range(E):
+                s[f"{p}.mlp.e{e}.gate"] = s[f"{p}.mlp.e{e}.up"] = (ff, W)
+                s[f"{p}.mlp.e{e}.down"] = (W, ff)
+            s[f"{p}.mlp.router"], s[f"{p}.mlp.router.b"] = (E, W), (E,)
+    return s
+
+
+def random_weights(cfg: dict, seed: int = 0, dtype=torch.float64, rank_a: int = 6, rank_g: int = 10) -> Dict[str, torch.Tensor]:
+    """weights that keep every mechanism visible in the logits; values are exactly representable in bfloat16"""
+    g = torch.Generator().manual_seed(seed)
+    w = {}
+    for name, shape in tensor_shapes(cfg, rank_a, rank_g).items():
+        leaf = name.split(".", 1)[1] if name.startswith("l") and "." in name else name
+        if name == "embed":
+            t = torch.randn(shape, generator=g) * 0.5
+        elif leaf.endswith(".conv"):
+            t = torch.randn(shape, generator=g) * 0.6
+        elif leaf.endswith("router"):
+            t = torch.randn(shape, generator=g) * (4.0 / math.sqrt(shape[1]))          # clear choices
+        elif len(shape) == 2:
+            t = torch.randn(shape, generator=g) * (1.5 / math.sqrt(shape[1]))
+        elif leaf.endswith("norm") or leaf.endswith("norm1") or leaf.endswith("norm2") or leaf.endswith(".out"):
+            t = 1.0 + 0.3 * torch.randn(shape, generator=g)
+        elif leaf.endswith("temp"):
+            t = 0.5 + torch.rand(shape, generator=g) * 3.0
+        elif leaf.endswith("vmix"):
+            t = torch.rand(shape, generator=g) * 0.8 + 0.1
+        elif leaf.endswith("A_log"):
+            t = torch.randn(shape, generator=g) * 0.7 - 1.0
+        elif leaf.endswith("dt_bias"):
+            t = torch.randn(shape, generator=g) - 1.0
+        elif leaf.endswith(".D"):
+            t = 1.0 + 0.5 * torch.randn(shape, generator=g)
+        elif leaf.endswith("pb"):
+            t = torch.randn(shape, generator=g) - 1.0
+        else:
+            t = torch.randn(shape, generator=g) * 0.5
+        w[name] = t.to(torch.bfloat16).to(dtype)
+    return w
