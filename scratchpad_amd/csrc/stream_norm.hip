@@ -338,6 +338,129 @@ add_group_norm_kernel(float* x, int64_t x_stride, const void* a, int64_t a_strid
     E::store(out_next, t * next_stride + i, rowbuf[i] * ginv[i / per] * next_weight[i]);
 }
 
+// The same on 16-byte vectors, for rows of NV x 256 vectors at most whose groups are whole vectors: a thread holds its part
+// of the row in registers; the vectors' sums of squares meet in LDS, where a wave per group adds them in a fixed order.
+template <typename Tag, int NV>
+__global__ void __launch_bounds__(kBlock)
+add_group_norm_vec_kernel(float* x, int64_t x_stride, const void* a, int64_t a_stride, const float* wa, const void* b,
+                          int64_t b_stride, const float* wb, void* out_next, int64_t next_stride, const float* next_weight,
+                          int width, int groups, float eps) {
+  typedef Elem<Tag> E;
+  constexpr int V = E::kVec;
+  __shared__ float red[2 * (kBlock / 64)];
+  __shared__ float vsq[NV * kBlock];
+  __shared__ float ginv[64];
+  const int64_t t = blockIdx.x;
+  const int nvec = width / V;
+  float ya[NV][V], yb[NV][V], xs[NV][V];
+#pragma unroll
+  for (int u = 0; u < NV; ++u) {
+    const int vi = threadIdx.x + u * kBlock;
+    const int64_t c = (int64_t)vi * V;
+    if (vi < nvec) {
+      if (a) unpack16<Tag>(ld16((const char*)a + (t * a_stride + c) * E::kBytes), ya[u]);
+      if (b) unpack16<Tag>(ld16((const char*)b + (t * b_stride + c) * E::kBytes), yb[u]);
+#pragma unroll
+      for (int q = 0; q < V / 4; ++q) unpack16<f32_tag>(ld16(x + t * x_stride + c + 4 * q), xs[u] + 4 * q);
+    }
+    if (vi >= nvec || !a) {
+#pragma unroll
+      for (int e = 0; e < V; ++e) ya[u][e] = 0.f;
+    }
+    if (vi >= nvec || !b) {
+#pragma unroll
+      for (int e = 0; e < V; ++e) yb[u][e] = 0.f;
+    }
+    if (vi >= nvec) {
+#pragma unroll
+      for (int e = 0; e < V; ++e) xs[u][e] = 0.f;
+    }
+  }
+  auto row4 = [&](const float* w, int64_t c, float* f) { unpack16<f32_tag>(ld16(w + c), f); };
+  if (b) {
+    float sa = 0.f, sb = 0.f;
+#pragma unroll
+    for (int u = 0; u < NV; ++u)
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        sa += ya[u][e] * ya[u][e];
+        sb += yb[u][e] * yb[u][e];
+      }
+    sa = wave_sum(sa);
+    sb = wave_sum(sb);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) {
+      red[2 * wave] = sa;
+      red[2 * wave + 1] = sb;
+    }
+    __syncthreads();
+    sa = sb = 0.f;
+    for (int w = 0; w < kBlock / 64; ++w) {
+      sa += red[2 * w];
+      sb += red[2 * w + 1];
+    }
+    const float ia = 1.f / sqrtf(sa / (float)width + eps), ib = 1.f / sqrtf(sb / (float)width + eps);
+#pragma unroll
+    for (int u = 0; u < NV; ++u) {
+      const int vi = threadIdx.x + u * kBlock;
+      if (vi < nvec) {
+#pragma unroll
+        for (int q = 0; q < V / 4; ++q) {
+          float fa[4], fb[4];
+          row4(wa, (int64_t)vi * V + 4 * q, fa);
+          row4(wb, (int64_t)vi * V + 4 * q, fb);
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            ya[u][4 * q + e] = 0.5f * (ya[u][4 * q + e] * ia * fa[e] + yb[u][4 * q + e] * ib * fb[e]);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < NV; ++u) {
+    const int vi = threadIdx.x + u * kBlock;
+    float sq = 0.f;
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      xs[u][e] += ya[u][e];
+      sq += xs[u][e] * xs[u][e];
+    }
+    if (vi < nvec) {
+      vsq[vi] = sq;
+      if (a) {
+#pragma unroll
+        for (int q = 0; q < V / 4; ++q) st16(x + t * x_stride + (int64_t)vi * V + 4 * q, pack16<f32_tag>(xs[u] + 4 * q));
+      }
+    }
+  }
+  if (!out_next) return;
+  __syncthreads();
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, pv = nvec / groups;      // vectors per group
+  for (int g = wave; g < groups; g += kBlock / 64) {
+    float ss = 0.f;
+    for (int i = lane; i < pv; i += 64) ss += vsq[g * pv + i];
+    ss = wave_sum(ss);
+    if (lane == 0) ginv[g] = 1.f / sqrtf(ss / (float)(pv * V) + eps);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < NV; ++u) {
+    const int vi = threadIdx.x + u * kBlock;
+    if (vi < nvec) {
+      const float inv = ginv[vi / pv];
+      float o[V];
+#pragma unroll
+      for (int q = 0; q < V / 4; ++q) {
+        float fw[4];
+        row4(next_weight, (int64_t)vi * V + 4 * q, fw);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[4 * q + e] = xs[u][4 * q + e] * inv * fw[e];
+      }
+      st16((char*)out_next + (t * next_stride + (int64_t)vi * V) * E::kBytes, pack16<Tag>(o));
+    }
+  }
+}
+
 }  // namespace
 }  // namespace sp
 
@@ -448,6 +571,26 @@ extern "C" int sp_add_group_norm(float* x, int64_t x_stride, const void* a, int6
   SP_CHECK_ARG(!a || a_stride >= width);
   SP_CHECK_ARG(!b || (a && wa && wb && b_stride >= width));
   SP_CHECK_ARG(!out_next || (next_weight && next_stride >= width));
+  // rows of 16-byte vectors that 256 threads hold in registers, groups of whole vectors: the vector kernel
+  const int vecn = dtype == SP_F32 ? 4 : 8, esize = dtype == SP_F32 ? 4 : 2;
+  auto al = [&](const void* p, int64_t stride, int elem_bytes) {
+    return !p || ((((uintptr_t)p) & 15) == 0 && (stride * elem_bytes) % 16 == 0);
+  };
+  if (width % vecn == 0 && (width / groups) % vecn == 0 && width / vecn <= 4 * kBlock && al(x, x_stride, 4) &&
+      al(a, a_stride, esize) && al(b, b_stride, esize) && al(out_next, next_stride, esize) && al(wa, 0, 4) && al(wb, 0, 4) &&
+      al(next_weight, 0, 4)) {
+    const int nv = (width / vecn + kBlock - 1) / kBlock;
+#define SP_AGN(NV)                                                                                                      \
+  SP_DISPATCH_DTYPE(dtype, (add_group_norm_vec_kernel<Tag, NV><<<dim3((unsigned)num_tokens), kBlock, 0, (hipStream_t)stream>>>( \
+                               x, x_stride, a, a_stride, wa, b, b_stride, wb, out_next, next_stride, next_weight, width, groups, \
+                               eps)))
+    if (nv <= 1) SP_AGN(1);
+    else if (nv <= 2) SP_AGN(2);
+    else SP_AGN(4);
+#undef SP_AGN
+    SP_LAUNCH_CHECK();
+    return SP_OK;
+  }
   SP_DISPATCH_DTYPE(dtype, (add_group_norm_kernel<Tag><<<dim3((unsigned)num_tokens), kBlock,
                                                           (size_t)(width + groups) * sizeof(float), (hipStream_t)stream>>>(
                                x, x_stride, a, a_stride, wa, b, b_stride, wb, out_next, next_stride, next_weight, width,
